@@ -105,10 +105,18 @@ _KERNEL_API = {
     "pa_sample_wide_workspace": (c_long, [I, I]),
     "pa_logprobs": (I, [P, P, P, P, P, P, P, I, I, I, I]),
     "pa_sample_wide": (I, [P, P, P, P, P, P, P, P, I, I, I]),
+    "pa_group_norm_step": (I, [P, I, P, P, P, P, P, P, I, I, I, F]),
+    "pa_poly_norm": (I, [P, I, P, P, P, P, I, I, F]),
+    "pa_head_norm_gate": (I, [P, I, P, P, c_long, P, P, c_long, I, I, I, F, I, F]),
+    "pa_attn_masked": (I, [P, I, P, P, P, P, I, P, P, P, c_long, I, I, I, I, I, I, I, I, F, F, P, P, P, c_long, F]),
+    "pa_qkv_prepare": (I, [P, I, P, c_long, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, F]),
+    "pa_delta_prepare": (I, [P, I, P, c_long, I, I, P, I, P, P, P, P, P, c_long, I, P, P, P, P, P, I, I, I, I, I, I]),
+    "pa_gated_delta": (I, [P, P, P, P, P, P, P, P, I, I, I, I, I]),
+    "pa_rotate_halves_f32": (I, [P, I, P, c_long, I, I, I, P, P, P, I, I, I, I, I, F]),
 }
 
 _HOST_API = {
-    "pa_cache_create": (P, [I, I, IP, IP, I]),
+    "pa_cache_create": (P, [I, I, IP, IP, IP, I]),
     "pa_cache_destroy": (None, [P]),
     "pa_cache_open": (I, [P, c_longlong, I]),
     "pa_cache_reserve": (I, [P, c_longlong, I]),

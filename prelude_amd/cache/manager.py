@@ -42,21 +42,25 @@ def _p(a: np.ndarray):
 class PageTables:
     """Pools, per-request tables and state slots (host side only; no GPU needed)."""
 
-    def __init__(self, page_size: int, groups: Sequence[Tuple[int, int]], state_slots: int = 0):
-        """``groups``: (number of pages, window or 0) per group."""
+    def __init__(self, page_size: int, groups: Sequence[Tuple[int, ...]], state_slots: int = 0):
+        """``groups``: (number of pages, window or 0[, first positions a window keeps]) per group."""
         if page_size < 1:
             raise CacheError(f"page size {page_size} must be positive")
-        for n, w in groups:
-            if n < 1 or w < 0:
-                raise CacheError(f"a cache group needs at least one page and a window >= 0, got ({n}, {w})")
+        groups = [(int(g[0]), int(g[1]), int(g[2]) if len(g) > 2 else 0) for g in groups]
+        for n, w, k in groups:
+            if n < 1 or w < 0 or k < 0:
+                raise CacheError(f"a cache group needs at least one page, a window >= 0 and kept first positions >= 0, "
+                                 f"got ({n}, {w}, {k})")
             if n * page_size >= 2 ** 31:
                 raise CacheError(f"{n} pages of {page_size} tokens exceed 32-bit slot numbers")
         self._lib = host()
         self.page_size = int(page_size)
-        self.groups = [(int(n), int(w)) for n, w in groups]
-        n = (ctypes.c_int * len(groups))(*[g[0] for g in self.groups])
-        w = (ctypes.c_int * len(groups))(*[g[1] for g in self.groups])
-        self._h = self._lib.pa_cache_create(self.page_size, len(self.groups), n, w, int(state_slots))
+        self.groups = [(n, w) for n, w, _ in groups]
+        self.keep_first = [k for _, _, k in groups]
+        n = (ctypes.c_int * len(groups))(*[g[0] for g in groups])
+        w = (ctypes.c_int * len(groups))(*[g[1] for g in groups])
+        k = (ctypes.c_int * len(groups))(*[g[2] for g in groups])
+        self._h = self._lib.pa_cache_create(self.page_size, len(self.groups), n, w, k, int(state_slots))
         if not self._h:
             raise CacheError("cache manager could not be created")
 
@@ -207,13 +211,14 @@ def state_bytes_per_slot(cache_specs: Sequence[object]) -> int:
     return sum(int(cs.bytes_per_slot()) for cs in cache_specs if not _paged(cs))
 
 
-def peak_pages(total: int, chunk: int, window: int, page_size: int) -> int:
+def peak_pages(total: int, chunk: int, window: int, page_size: int, keep_first: int = 0) -> int:
     """Pages of a group with this window that a request of ``total`` tokens holds at most when it is fed in
-    portions of at most ``chunk`` tokens (the rule of ``CacheManager::peak_pages``)."""
+    portions of at most ``chunk`` tokens (the rule of ``CacheManager::peak_pages``); the pages of the first
+    ``keep_first`` positions are held throughout."""
     pages = lambda n: -(-n // page_size)
     if window <= 0:
         return pages(total)
-    return min(pages(total), pages(max(1, chunk) + window - 1) + 1)
+    return min(pages(total), pages(max(1, chunk) + window - 1) + 1 + (pages(keep_first) if keep_first > 0 else 0))
 
 
 def pages_per_group(tokens: int, group_specs: Sequence[PagedCacheSpec], page_size: int, max_requests: int,
@@ -225,7 +230,8 @@ def pages_per_group(tokens: int, group_specs: Sequence[PagedCacheSpec], page_siz
     out = []
     for g in group_specs:
         if g.window > 0:
-            out.append(max(1, min(full, max_requests * peak_pages(max_request_tokens, chunk, g.window, page_size))))
+            out.append(max(1, min(full, max_requests * peak_pages(max_request_tokens, chunk, g.window, page_size,
+                                                                  int(getattr(g, "keep_first", 0))))))
         else:
             out.append(full)
     return out

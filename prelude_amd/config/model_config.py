@@ -447,3 +447,185 @@ class FazopelConfig:
         norm = _obj(raw, "norm", a)
         return cls(vocab=_positive(raw, "vocab", int, a, ""), width=_positive(raw, "width", int, a, ""),
                    norm_eps=_positive(norm, "eps", float, a, "norm."), layers=tuple(layers))
+
+
+# ---------------------------------------------------------------------------
+@dataclasses.dataclass(frozen=True)
+class WindowMask:
+    size: int          # the query at i sees the key at j <= i with i - j < size; 0: every earlier key
+    keep_first: int    # ... or j < keep_first
+
+
+@dataclasses.dataclass(frozen=True)
+class TedalixAttentionConfig:
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    mask: WindowMask
+    softcap: float = 0.0              # the sink mixer only; 0: none
+    kv_from: Optional[int] = None     # the layer whose cached keys and values this one reads
+
+
+@dataclasses.dataclass(frozen=True)
+class TedalixDeltaConfig:
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+    rank: Optional[int]     # inner size of the two-step projections; None: what the tensors have
+
+
+@dataclasses.dataclass(frozen=True)
+class TedalixParallelConfig:
+    left: TedalixAttentionConfig
+    right: TedalixDeltaConfig
+    left_scale: float
+    right_scale: float
+
+
+@dataclasses.dataclass(frozen=True)
+class TedalixRetentionConfig:
+    heads: int
+    dim: int
+    vdim: int
+    decay: Tuple[float, ...]
+    rot_base: float
+    rot_dims: int           # 0: no rotation
+
+
+@dataclasses.dataclass(frozen=True)
+class TedalixLayerConfig:
+    type: str               # "attention" | "parallel" | "retention"
+    mixer: object
+    ff: int                 # inner size of the dense feed-forward; 0: the layer has none
+
+
+@dataclasses.dataclass(frozen=True)
+class TedalixConfig:
+    """Tedalix: a decoder whose layers are listed one by one in ``layers``, each with a norm in front of and behind
+    every branch (RMS norms in ``norm.groups`` groups).  A layer's mixer is attention under a window that keeps the
+    first tokens (``attention``; it may read another layer's cached keys and values, ``kv_from``), attention with a
+    sink, capped scores, a bias by distance and a gate per head beside the gated delta rule (``parallel``), or linear
+    attention with a fixed decay per head and rotary positions (``retention``).  The feed-forward is dense with the
+    polynomial activation, or absent.  Every size and constant is read from here; there is no longest position and
+    no end-of-sequence id."""
+    vocab: int
+    width: int
+    norm_eps: float
+    norm_groups: int
+    layers: Tuple[TedalixLayerConfig, ...]
+
+    ARCH = "Tedalix"
+    MIXERS = ("attention", "parallel", "retention")
+
+    @classmethod
+    def _mask(cls, m: Mapping[str, Any], mw: str) -> WindowMask:
+        a = cls.ARCH
+        mask = _obj(m, "mask", a, mw, optional=True)
+        if mask is None:
+            return WindowMask(0, 0)
+        size = _positive(mask, "size", int, a, mw + "mask.")
+        try:
+            keep = _get(mask, "keep_first", int, a, default=0)
+        except ConfigError as e:
+            raise ConfigError(str(e).replace("`keep_first`", f"`{mw}mask.keep_first`")) from None
+        return WindowMask(size, keep)
+
+    @classmethod
+    def _attention(cls, m: Mapping[str, Any], mw: str, sink: bool) -> TedalixAttentionConfig:
+        a = cls.ARCH
+        heads, kv_heads = _positive(m, "heads", int, a, mw), _positive(m, "kv_heads", int, a, mw)
+        if heads % kv_heads:
+            raise ConfigError(f"failed to parse {a} config: `{mw}heads` ({heads}) is no multiple of `kv_heads` ({kv_heads})")
+        softcap = 0.0
+        if sink and m.get("softcap") is not None:
+            softcap = _positive(m, "softcap", float, a, mw)
+        src = None
+        if not sink and m.get("kv_from") is not None:
+            try:
+                src = _get(m, "kv_from", int, a)
+            except ConfigError as e:
+                raise ConfigError(str(e).replace("`kv_from`", f"`{mw}kv_from`")) from None
+        return TedalixAttentionConfig(heads, kv_heads, _positive(m, "dim", int, a, mw), _positive(m, "vdim", int, a, mw),
+                                      _positive(m, "scale", float, a, mw), cls._mask(m, mw), softcap, src)
+
+    @classmethod
+    def _mixer(cls, kind: str, m: Mapping[str, Any], mw: str):
+        a = cls.ARCH
+        if kind == "attention":
+            return cls._attention(m, mw, sink=False)
+        if kind == "parallel":
+            r = _obj(m, "right", a, mw)
+            rw = mw + "right."
+            heads, kv_heads = _positive(r, "heads", int, a, rw), _positive(r, "kv_heads", int, a, rw)
+            if heads % kv_heads:
+                raise ConfigError(f"failed to parse {a} config: `{rw}heads` ({heads}) is no multiple of `kv_heads` ({kv_heads})")
+            rank = _positive(r, "rank", int, a, rw) if r.get("rank") is not None else None
+            right = TedalixDeltaConfig(heads, kv_heads, _positive(r, "dim", int, a, rw), _positive(r, "vdim", int, a, rw),
+                                       _positive(r, "conv", int, a, rw), rank)
+            try:
+                ls, rs = _get(m, "left_scale", float, a), _get(m, "right_scale", float, a)
+            except ConfigError as e:
+                raise ConfigError(str(e).replace("`left_scale`", f"`{mw}left_scale`").replace("`right_scale`", f"`{mw}right_scale`")) from None
+            return TedalixParallelConfig(cls._attention(_obj(m, "left", a, mw), mw + "left.", sink=True), right, ls, rs)
+        heads = _positive(m, "heads", int, a, mw)
+        decay = m.get("decay")
+        if not isinstance(decay, list) or len(decay) != heads or \
+                not all(isinstance(x, (int, float)) and not isinstance(x, bool) and 0.0 <= x <= 1.0 for x in decay):
+            raise ConfigError(f"failed to parse {a} config: `{mw}decay` must list one number in [0, 1] for each of the "
+                              f"{heads} heads, got {decay!r}")
+        dim = _positive(m, "dim", int, a, mw)
+        rot = _obj(m, "rot", a, mw, optional=True)
+        base, dims = 1.0, 0
+        if rot is not None:
+            base, dims = _positive(rot, "base", float, a, mw + "rot."), _positive(rot, "dims", int, a, mw + "rot.")
+            if dims % 2 or dims > dim:
+                raise ConfigError(f"failed to parse {a} config: `{mw}rot.dims` ({dims}) must be even and at most `dim` ({dim})")
+        return TedalixRetentionConfig(heads, dim, _positive(m, "vdim", int, a, mw), tuple(float(x) for x in decay), base, dims)
+
+    @classmethod
+    def from_dict(cls, raw: Mapping[str, Any]) -> "TedalixConfig":
+        a = cls.ARCH
+        layers_raw = raw.get("layers")
+        if not isinstance(layers_raw, list) or not layers_raw:
+            raise ConfigError(f"failed to parse {a} config: `layers` must be a non-empty list")
+        layers = []
+        for i, lr in enumerate(layers_raw):
+            w = f"layers[{i}]."
+            if not isinstance(lr, dict):
+                raise ConfigError(f"failed to parse {a} config: `layers[{i}]` must be an object")
+            kind = _get(lr, "type", str, a)
+            if kind not in cls.MIXERS:
+                raise ConfigError(f"failed to parse {a} config: `{w}type` {kind!r} is not one of {list(cls.MIXERS)}")
+            f = _obj(lr, "mlp", a, w, optional=True)
+            ff = 0
+            if f is not None:
+                fk = _get(f, "kind", str, a)
+                if fk != "dense":
+                    raise ConfigError(f"failed to parse {a} config: `{w}mlp.kind` {fk!r} is not one of ['dense']")
+                ff = _positive(f, "ff", int, a, w + "mlp.")
+            layers.append(TedalixLayerConfig(kind, cls._mixer(kind, _obj(lr, "mixer", a, w), w + "mixer."), ff))
+        for i, layer in enumerate(layers):
+            src = layer.mixer.kv_from if layer.type == "attention" else None
+            if src is None:
+                continue
+            w = f"layers[{i}].mixer."
+            if not 0 <= src < len(layers) or src == i or layers[src].type != "attention" or layers[src].mixer.kv_from is not None:
+                raise ConfigError(f"failed to parse {a} config: `{w}kv_from` ({src}) must name another attention layer that "
+                                  f"has keys and values of its own")
+            if src > i:
+                raise ConfigError(f"failed to parse {a} config: `{w}kv_from` ({src}) names a layer that runs later")
+            m, o = layer.mixer, layers[src].mixer
+            if (m.kv_heads, m.dim, m.vdim) != (o.kv_heads, o.dim, o.vdim):
+                raise ConfigError(f"failed to parse {a} config: `{w}kv_heads`, `dim` and `vdim` must equal those of layer {src}, "
+                                  f"whose keys and values it reads")
+        norm = _obj(raw, "norm", a)
+        width = _positive(raw, "width", int, a, "")
+        groups = _positive(norm, "groups", int, a, "norm.") if norm.get("groups") is not None else 1
+        if width % groups:
+            raise ConfigError(f"failed to parse {a} config: `norm.groups` ({groups}) does not divide `width` ({width})")
+        return cls(vocab=_positive(raw, "vocab", int, a, ""), width=width, norm_eps=_positive(norm, "eps", float, a, "norm."),
+                   norm_groups=groups, layers=tuple(layers))

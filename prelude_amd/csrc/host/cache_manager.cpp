@@ -173,6 +173,11 @@ int CacheManager::first_key_needed(int g, int start) const {
   return std::max(0, start - w + 1);
 }
 
+int CacheManager::kept_pages(int g) const {
+  if (groups_[g].window <= 0 || groups_[g].keep_first <= 0) return 0;
+  return table_len(groups_[g].keep_first);
+}
+
 int CacheManager::pages_needed(int64_t id, int new_len, int g) const {
   const RequestCache* rc = find(id);
   const int want = table_len(new_len);
@@ -186,7 +191,7 @@ int CacheManager::peak_pages(int total, int chunk, int g) const {
   if (w <= 0) return all;
   // a portion of `chunk` tokens sees back over w - 1 keys; one more page for the misalignment at either end
   const int span = table_len(std::max(1, chunk) + w - 1) + 1;
-  return std::min(all, span);
+  return std::min(all, span + kept_pages(g));
 }
 
 int CacheManager::live_pages(int64_t id, int g) const {
@@ -205,7 +210,7 @@ int CacheManager::reservable_len(int64_t id) const {
     const auto& table = rc->tables[g];
     const int first_key = first_key_needed(g, rc->len);
     int releasable = 0;
-    for (int i = rc->first_live[g]; i < (int)table.size() && (i + 1) * page_size_ <= first_key; ++i)
+    for (int i = std::max(rc->first_live[g], kept_pages(g)); i < (int)table.size() && (i + 1) * page_size_ <= first_key; ++i)
       releasable += table[i] >= 0;
     const long reach = ((long)table.size() + pools_[g].free_count() + releasable) * page_size_;
     if (best < 0 || reach < best) best = reach;
@@ -217,6 +222,7 @@ int CacheManager::reservable_len(int64_t id) const {
 void CacheManager::release_before(RequestCache& rc, int g, int first_key) {
   auto& table = rc.tables[g];
   int& i = rc.first_live[g];
+  i = std::max(i, kept_pages(g));   // the pages of the kept first positions stay
   while (i < (int)table.size() && (i + 1) * page_size_ <= first_key) {
     if (table[i] >= 0) {
       pools_[g].give(table[i]);

@@ -24,6 +24,8 @@ namespace pa {
 struct GroupSpec {
   int num_pages = 0;
   int window = 0;  // keys a layer of this group looks back over, the query's own included; 0 = all
+  int keep_first = 0;  // with a window: the first positions stay visible to every later token, so the pages that hold them
+                       // are never given back while the request lives
 };
 
 // A fixed set of pages.  A page goes to whoever asks, first-in first-out, but a request's pages are kept in runs
@@ -150,6 +152,7 @@ class CacheManager {
  private:
   void release_before(RequestCache& rc, int g, int first_key_needed);
   int first_key_needed(int g, int start) const;
+  int kept_pages(int g) const;   // pages at a request's start that a window never passes
 
   int page_size_;
   std::vector<GroupSpec> groups_;

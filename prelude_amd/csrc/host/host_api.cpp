@@ -24,12 +24,14 @@ struct SchedHandle {
 
 extern "C" {
 
-void* pa_cache_create(int page_size, int n_groups, const int* num_pages, const int* windows, int state_slots) {
+void* pa_cache_create(int page_size, int n_groups, const int* num_pages, const int* windows, const int* keep_first,
+                      int state_slots) {
   if (page_size < 1 || n_groups < 0) return nullptr;
   std::vector<pa::GroupSpec> groups(n_groups);
   for (int g = 0; g < n_groups; ++g) {
     groups[g].num_pages = num_pages[g];
     groups[g].window = windows[g];
+    groups[g].keep_first = keep_first ? keep_first[g] : 0;
   }
   return new CacheHandle(page_size, groups, state_slots);
 }

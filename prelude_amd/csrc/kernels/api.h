@@ -282,6 +282,40 @@ int pa_moe_linear_mfma(void* stream, int y_dtype, const void* x, const void* w, 
 int pa_head_linear_mfma(void* stream, const void* x, const void* w, void* y, int tokens, int heads, int K, int N, long xs_t,
                         long xs_h, long ys_t, long ys_h);
 
+// ---- statistics over parts of a row (rowwise_groups.hip) ----
+// Around a 32-bit stream: with y, residual[r] += norm_g(y[r]) * w_add; with out, out[r] = norm_g(residual[row]) * w_out
+// (row = rows[r] when rows is given, which goes without y).  norm_g: the row in `groups` equal consecutive parts, each
+// over its own sqrt(mean(part^2) + eps).
+int pa_group_norm_step(void* stream, int dtype, const void* y, const float* w_add, float* residual, const float* w_out,
+                       void* out, const int* rows, int nrows, int hidden, int groups, float eps);
+// out = a N(z) + b N(z^2) + c N(z^3) + e, z = x (+ bias), N(u) = u / sqrt(mean(u^2) + eps) over the row; coeff (a, b, c, e).
+int pa_poly_norm(void* stream, int dtype, const void* x, const float* bias, const float* coeff, void* out, int nrows,
+                 int width, float eps);
+// out[r, h, :] = o[r, h, :] / sqrt(mean(o[r, h, :]^2) + eps) * w (null: none; vdim elements shared by the heads)
+//                * act(gate[r, h, :]) * scale;  act 0 sigmoid, 1 silu.
+int pa_head_norm_gate(void* stream, int dtype, const float* o, const void* gate, long gate_stride, const float* w, void* out,
+                      long out_stride, int nrows, int heads, int vdim, float eps, int act, float scale);
+
+// ---- attention with a window that keeps first tokens, a bias by distance, a gate a head (attention_masked.hip) ----
+int pa_attn_masked(void* stream, int dtype, const void* q, const void* k_cache, const void* v_cache, const int* block_table,
+                   int table_stride, const int* seq_of_token, const int* positions, void* out, long out_stride, int tokens,
+                   int nh, int nkv, int hd, int vd, int page_size, int window, int keep_first, float scale, float softcap,
+                   const float* slopes, const float* sink, const void* gate, long gate_stride, float out_scale);
+int pa_qkv_prepare(void* stream, int dtype, const void* p, long stride, int q_off, int k_off, int v_off, const float* qw,
+                   const float* kw, const int* slots, void* q_out, void* k_cache, void* v_cache, int tokens, int nh, int nkv,
+                   int hd, int vd, int page_size, float eps);
+
+// ---- the gated delta rule and what stands in front of a recurrence (delta_rule.hip) ----
+int pa_delta_prepare(void* stream, int dtype, const void* p, long stride, int off, int b_off, const float* w, int taps,
+                     float* conv_state, const int* seq_of_token, const int* cu_q, const int* state_slots, const void* a,
+                     long a_stride, int a_off, const float* a_log, const float* dt_bias, float* out, float* decay, float* beta,
+                     int tokens, int nseq, int heads, int kvh, int d, int e);
+int pa_gated_delta(void* stream, const float* x, const float* decay, const float* beta, float* state, const int* state_slots,
+                   const int* cu_q, float* out, int nseq, int heads, int kvh, int d, int e);
+int pa_rotate_halves_f32(void* stream, int dtype, const void* p, long stride, int q_off, int k_off, int v_off,
+                         const float* inv_freq, const int* positions, float* out, int tokens, int heads, int d, int e, int rot,
+                         float k_scale);
+
 #ifdef __cplusplus
 }
 #endif

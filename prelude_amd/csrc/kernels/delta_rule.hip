@@ -1,0 +1,269 @@
+// The gated delta rule, a recurrent mixer with a state of fixed size per request, and what stands in front of a
+// recurrence: a short causal convolution per channel with its own carried inputs, unit vectors per head, decays from
+// a softplus, and (for linear attention with rotary positions) the rotation of queries and keys in 32-bit.
+//
+// Per head, with unit vectors q, k [d] (q also times d^(-1/2)), values v [e], a gate beta and a decay g [d] per key
+// channel, the state S [d, e] (32-bit, zero at a request's start) moves token by token:
+//
+//     S <- diag(g) S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q
+//
+// so the read-out sees the token's own write.  Everything here is 32-bit; the order of every sum follows the token's
+// place alone, so outputs and state are the same bits however a prompt is cut into steps.
+#include "common.h"
+#include "api.h"
+
+namespace pa {
+
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
+__device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+
+// A workgroup a token.  p [T, stride] holds, from column `off`, the channels [qk | qk | vv] (queries and keys of
+// `kvh` heads of d, values of `heads` heads of e).  Every channel c: y_t = silu(sum_s w[c, s] x_(t - (taps - 1 - s))),
+// inputs before the step's first token of the sequence from conv_state [slots, C, taps - 1] (oldest first; zero for
+// a request that starts).  Then queries and keys become unit vectors per head (x / sqrt(sum x^2 + 1e-6)), the
+// queries also times d^(-1/2).  out [T, C] 32-bit.  Also: decay [T, heads * d] = exp(-exp(a_log[h]) *
+// softplus(a[t, h * d + j] + dt_bias[h * d + j])) from a [T, a_stride] at column a_off, and beta [T, heads] =
+// sigmoid(b[t, h]) from p at column b_off.
+template <typename T>
+__global__ __launch_bounds__(256) void delta_prepare_kernel(
+    const T* __restrict__ p, size_t stride, int off, int b_off, const float* __restrict__ w, int taps,
+    const float* __restrict__ conv_state, const int* __restrict__ seq_of_token, const int* __restrict__ cu_q,
+    const int* __restrict__ state_slots, const T* __restrict__ a, size_t a_stride, int a_off,
+    const float* __restrict__ a_log, const float* __restrict__ dt_bias, float* __restrict__ out,
+    float* __restrict__ decay, float* __restrict__ beta, int heads, int kvh, int d, int e) {
+  extern __shared__ float y[];
+  const int t = blockIdx.x;
+  const int seq = seq_of_token[t];
+  const int local = t - cu_q[seq];          // tokens of this sequence in the step before this one
+  const int slot = state_slots[seq];
+  const int qk = kvh * d, C = 2 * qk + heads * e;
+  const float* st = conv_state + (size_t)slot * C * (taps - 1);
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    float acc = 0.f;
+    for (int s = 0; s < taps; ++s) {
+      const int back = taps - 1 - s;          // how many tokens back this tap reaches
+      float x;
+      if (back <= local) x = to_f32(p[(size_t)(t - back) * stride + off + c]);
+      else x = st[(size_t)c * (taps - 1) + (taps - 1) - (back - local)];
+      acc = fmaf(w[(size_t)c * taps + s], x, acc);
+    }
+    y[c] = silu_f(acc);
+  }
+  __syncthreads();
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave, nwaves = blockDim.x / kWave;
+  for (int v = wave; v < 2 * kvh; v += nwaves) {      // vectors to bring to unit length: kvh of q, then kvh of k
+    float ss = 0.f;
+    for (int j = lane; j < d; j += kWave) ss += y[v * d + j] * y[v * d + j];
+    ss = wave_sum(ss);
+    float f = 1.0f / sqrtf(ss + 1e-6f);
+    if (v < kvh) f *= 1.0f / sqrtf((float)d);
+    for (int j = lane; j < d; j += kWave) y[v * d + j] *= f;
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < C; c += blockDim.x) out[(size_t)t * C + c] = y[c];
+  for (int i = threadIdx.x; i < heads * d; i += blockDim.x) {
+    const float rate = expf(a_log[i / d]);
+    decay[(size_t)t * heads * d + i] = expf(-rate * softplus_f(to_f32(a[(size_t)t * a_stride + a_off + i]) + dt_bias[i]));
+  }
+  for (int h = threadIdx.x; h < heads; h += blockDim.x)
+    beta[(size_t)t * heads + h] = 1.0f / (1.0f + expf(-to_f32(p[(size_t)t * stride + b_off + h])));
+}
+
+// After the step's convolutions: a sequence's carried inputs become the last taps - 1 inputs it has seen.  A thread a
+// (sequence, channel); it reads all it needs before it writes.
+template <typename T>
+__global__ void conv_state_update_kernel(const T* __restrict__ p, size_t stride, int off, int C, int taps,
+                                         float* __restrict__ conv_state, const int* __restrict__ cu_q,
+                                         const int* __restrict__ state_slots, int nseq) {
+  const int seq = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C || seq >= nseq) return;
+  const int begin = cu_q[seq], n = cu_q[seq + 1] - begin;
+  if (n <= 0) return;
+  const int keep = taps - 1;
+  float* st = conv_state + ((size_t)state_slots[seq] * C + c) * keep;
+  float fresh[8];
+  for (int i = 0; i < keep; ++i) {
+    const int rel = n - keep + i;     // the step's token this place now holds, or an older one when negative
+    fresh[i] = rel >= 0 ? to_f32(p[(size_t)(begin + rel) * stride + off + c]) : st[i + n];
+  }
+  for (int i = 0; i < keep; ++i) st[i] = fresh[i];
+}
+
+// The recurrence.  A wavefront owns 64 value columns of one (sequence, head); a lane keeps its column of S in
+// registers (D rows, the key width rounded up).  Tokens are walked in order, a block of them staged in LDS.
+// x [T, C] 32-bit as delta_prepare left it ([q | k | v]), decay [T, heads, d], beta [T, heads];
+// state [slots, heads, d, e]; out [T, heads, e].
+template <int D>
+__global__ __launch_bounds__(kWave) void gated_delta_kernel(const float* __restrict__ x, const float* __restrict__ decay,
+                                                           const float* __restrict__ beta, float* __restrict__ state,
+                                                           const int* __restrict__ state_slots, const int* __restrict__ cu_q,
+                                                           float* __restrict__ out, int heads, int kvh, int d, int e) {
+  constexpr int NT = D <= 128 ? 16 : 8;
+  __shared__ float ks[NT][D], qs[NT][D], gs[NT][D];
+  __shared__ float bs[NT];
+  const int seq = blockIdx.x, h = blockIdx.y;
+  const int col = blockIdx.z * kWave + threadIdx.x;
+  const bool live = col < e;
+  const int begin = cu_q[seq], end = cu_q[seq + 1];
+  if (end <= begin) return;
+  const int kh = h / (heads / kvh);
+  const int qk = kvh * d, C = 2 * qk + heads * e;
+  float* S = state + (((size_t)state_slots[seq] * heads + h) * d) * e;
+  float s[D];
+#pragma unroll
+  for (int j = 0; j < D; ++j) s[j] = (live && j < d) ? S[(size_t)j * e + col] : 0.f;
+  for (int t0 = begin; t0 < end; t0 += NT) {
+    const int n = end - t0 < NT ? end - t0 : NT;
+    __syncthreads();
+    for (int i = threadIdx.x; i < n * D; i += kWave) {
+      const int tk = i / D, j = i % D;
+      const size_t t = t0 + tk;
+      const bool in = j < d;
+      qs[tk][j] = in ? x[t * C + kh * d + j] : 0.f;
+      ks[tk][j] = in ? x[t * C + qk + kh * d + j] : 0.f;
+      gs[tk][j] = in ? decay[(t * heads + h) * d + j] : 1.f;
+    }
+    if (threadIdx.x < n) bs[threadIdx.x] = beta[(size_t)(t0 + threadIdx.x) * heads + h];
+    __syncthreads();
+    float v[NT];
+#pragma unroll
+    for (int tk = 0; tk < NT; ++tk) v[tk] = (live && tk < n) ? x[(size_t)(t0 + tk) * C + 2 * qk + h * e + col] : 0.f;
+#pragma unroll
+    for (int tk = 0; tk < NT; ++tk) {
+      if (tk < n) {
+        float kv = 0.f;
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+          s[j] *= gs[tk][j];
+          kv = fmaf(s[j], ks[tk][j], kv);
+        }
+        const float u = bs[tk] * (v[tk] - kv);
+        float o = 0.f;
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+          s[j] = fmaf(ks[tk][j], u, s[j]);
+          o = fmaf(s[j], qs[tk][j], o);
+        }
+        if (live) out[((size_t)(t0 + tk) * heads + h) * e + col] = o;
+      }
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int j = 0; j < D; ++j)
+      if (j < d) S[(size_t)j * e + col] = s[j];
+  }
+}
+
+// p [T, stride] -> out [T, 2 * heads * d + heads * e] 32-bit: queries (from q_off) and keys (from k_off) with the
+// first `rot` dimensions of every head turned, dimension i with i + rot / 2, by positions[t] * inv_freq[i]; the keys
+// then times k_scale; values (from v_off) as they are.  A thread an element (a pair's two ends are two threads).
+template <typename T>
+__global__ void rotate_halves_f32_kernel(const T* __restrict__ p, size_t stride, int q_off, int k_off, int v_off,
+                                         const float* __restrict__ inv_freq, const int* __restrict__ positions,
+                                         float* __restrict__ out, int tokens, int heads, int d, int e, int rot, float k_scale) {
+  const int qk = heads * d, width = 2 * qk + heads * e;
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (size_t)tokens * width) return;
+  const size_t t = i / width;
+  const int c = (int)(i % width);
+  const T* row = p + t * stride;
+  if (c >= 2 * qk) {
+    out[i] = to_f32(row[v_off + c - 2 * qk]);
+    return;
+  }
+  const bool key = c >= qk;
+  const int base = key ? k_off : q_off;
+  const int cc = key ? c - qk : c;
+  const int j = cc % d;
+  float val = to_f32(row[base + cc]);
+  if (j < rot) {
+    const int half = rot / 2;
+    const int f = j < half ? j : j - half;
+    const float ang = (float)positions[t] * inv_freq[f];
+    const float cs = cosf(ang), sn = sinf(ang);
+    const float other = to_f32(row[base + cc + (j < half ? half : -half)]);
+    val = j < half ? val * cs - other * sn : val * cs + other * sn;
+  }
+  out[i] = key ? val * k_scale : val;
+}
+
+}  // namespace pa
+
+using namespace pa;
+
+extern "C" int pa_delta_prepare(void* stream, int dtype, const void* p, long stride, int off, int b_off, const float* w,
+                                int taps, float* conv_state, const int* seq_of_token, const int* cu_q, const int* state_slots,
+                                const void* a, long a_stride, int a_off, const float* a_log, const float* dt_bias, float* out,
+                                float* decay, float* beta, int tokens, int nseq, int heads, int kvh, int d, int e) {
+  if (tokens == 0) return 0;
+  PA_REQUIRE(tokens > 0 && nseq > 0 && heads > 0 && kvh > 0 && d > 0 && e > 0 && heads % kvh == 0,
+             "delta_prepare: bad sizes tokens=%d sequences=%d heads=%d key heads=%d d=%d e=%d", tokens, nseq, heads, kvh, d, e);
+  PA_REQUIRE(taps >= 1 && taps <= 9, "delta_prepare: a convolution of %d taps is outside 1..9", taps);
+  const long C = 2L * kvh * d + (long)heads * e;
+  PA_REQUIRE(C <= 15360, "delta_prepare: %ld channels are more than the 15360 the kernel takes", C);
+  PA_REQUIRE(off >= 0 && off + C <= stride && b_off >= 0 && b_off + heads <= stride && a_off >= 0 &&
+             a_off + (long)heads * d <= a_stride, "delta_prepare: the columns do not fit their rows");
+  hipStream_t st = (hipStream_t)stream;
+  const size_t lds = (size_t)C * sizeof(float);
+  if (dtype == kF32) {
+    hipLaunchKernelGGL(delta_prepare_kernel<float>, dim3(tokens), dim3(256), lds, st, (const float*)p, (size_t)stride, off,
+                       b_off, w, taps, conv_state, seq_of_token, cu_q, state_slots, (const float*)a, (size_t)a_stride, a_off,
+                       a_log, dt_bias, out, decay, beta, heads, kvh, d, e);
+    if (taps > 1)
+      hipLaunchKernelGGL(conv_state_update_kernel<float>, dim3((unsigned)((C + 255) / 256), nseq), dim3(256), 0, st,
+                         (const float*)p, (size_t)stride, off, (int)C, taps, conv_state, cu_q, state_slots, nseq);
+  } else if (dtype == kBF16) {
+    hipLaunchKernelGGL(delta_prepare_kernel<bf16>, dim3(tokens), dim3(256), lds, st, (const bf16*)p, (size_t)stride, off, b_off,
+                       w, taps, conv_state, seq_of_token, cu_q, state_slots, (const bf16*)a, (size_t)a_stride, a_off, a_log,
+                       dt_bias, out, decay, beta, heads, kvh, d, e);
+    if (taps > 1)
+      hipLaunchKernelGGL(conv_state_update_kernel<bf16>, dim3((unsigned)((C + 255) / 256), nseq), dim3(256), 0, st,
+                         (const bf16*)p, (size_t)stride, off, (int)C, taps, conv_state, cu_q, state_slots, nseq);
+  } else {
+    return pa::fail("delta_prepare: unknown element type code %d", dtype);
+  }
+  return check_launch("delta_prepare");
+}
+
+extern "C" int pa_gated_delta(void* stream, const float* x, const float* decay, const float* beta, float* state,
+                              const int* state_slots, const int* cu_q, float* out, int nseq, int heads, int kvh, int d, int e) {
+  if (nseq == 0) return 0;
+  PA_REQUIRE(nseq > 0 && heads > 0 && kvh > 0 && heads % kvh == 0 && d > 0 && e > 0,
+             "gated_delta: bad sizes sequences=%d heads=%d key heads=%d d=%d e=%d", nseq, heads, kvh, d, e);
+  PA_REQUIRE(d <= 256, "gated_delta: a key width of %d is more than the 256 the kernel takes", d);
+  dim3 grid(nseq, heads, (e + kWave - 1) / kWave);
+  hipStream_t st = (hipStream_t)stream;
+#define PA_DELTA(D) hipLaunchKernelGGL(gated_delta_kernel<D>, grid, dim3(kWave), 0, st, x, decay, beta, state, state_slots, cu_q, \
+                                       out, heads, kvh, d, e)
+  if (d <= 32) PA_DELTA(32);
+  else if (d <= 64) PA_DELTA(64);
+  else if (d <= 128) PA_DELTA(128);
+  else PA_DELTA(256);
+#undef PA_DELTA
+  return check_launch("gated_delta");
+}
+
+extern "C" int pa_rotate_halves_f32(void* stream, int dtype, const void* p, long stride, int q_off, int k_off, int v_off,
+                                    const float* inv_freq, const int* positions, float* out, int tokens, int heads, int d,
+                                    int e, int rot, float k_scale) {
+  if (tokens == 0) return 0;
+  PA_REQUIRE(tokens > 0 && heads > 0 && d > 0 && e > 0, "rotate_halves: bad sizes tokens=%d heads=%d d=%d e=%d", tokens, heads, d, e);
+  PA_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= d && (rot == 0 || inv_freq),
+             "rotate_halves: %d turned dimensions must be even, at most %d, and come with frequencies", rot, d);
+  PA_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && q_off + (long)heads * d <= stride && k_off + (long)heads * d <= stride &&
+             v_off + (long)heads * e <= stride, "rotate_halves: the columns do not fit the row of %ld", stride);
+  const long total = (long)tokens * (2L * heads * d + (long)heads * e);
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == kF32)
+    hipLaunchKernelGGL(rotate_halves_f32_kernel<float>, dim3(blocks), dim3(256), 0, st, (const float*)p, (size_t)stride, q_off,
+                       k_off, v_off, inv_freq, positions, out, tokens, heads, d, e, rot, k_scale);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(rotate_halves_f32_kernel<bf16>, dim3(blocks), dim3(256), 0, st, (const bf16*)p, (size_t)stride, q_off,
+                       k_off, v_off, inv_freq, positions, out, tokens, heads, d, e, rot, k_scale);
+  else
+    return pa::fail("rotate_halves: unknown element type code %d", dtype);
+  return check_launch("rotate_halves");
+}

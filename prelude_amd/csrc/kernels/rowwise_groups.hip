@@ -1,0 +1,194 @@
+// Row-wise kernels whose statistics are taken over parts of a row: the RMS norm in groups around a 32-bit stream,
+// the polynomial activation whose three powers are each brought to unit RMS, and the per-head norm with a gate that
+// follows a recurrent mixer.  All arithmetic is 32-bit; the order of every sum follows the thread layout alone, so a
+// row's result never depends on what else the launch holds.
+#include "common.h"
+#include "api.h"
+
+namespace pa {
+
+constexpr int kRowThreads = 256;
+
+// Sum of squares of part `g` (elements [g * len, (g + 1) * len)) of a row held in LDS.
+__device__ __forceinline__ float part_square_sum(const float* row, int g, int len, float* scratch) {
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < len; i += blockDim.x) {
+    const float v = row[g * len + i];
+    ss += v * v;
+  }
+  return block_sum(ss, scratch);
+}
+
+// One step around a stream kept in 32-bit, a workgroup a row:
+//   with y:      residual[r] += norm_g(y[r]) * w_add        (a branch's output normed in groups and added)
+//   with out:    out[r] = norm_g(residual[row]) * w_out     (the next branch's input, in the engine's type)
+// norm_g: the row in `groups` equal consecutive parts, each over its own sqrt(mean(part^2) + eps).
+// `rows` (only without y): output row r is the norm of residual row rows[r].
+template <typename T>
+__global__ __launch_bounds__(kRowThreads) void group_norm_step_kernel(
+    const T* __restrict__ y, const float* __restrict__ w_add, float* __restrict__ residual,
+    const float* __restrict__ w_out, T* __restrict__ out, const int* __restrict__ rows, int hidden, int groups, float eps) {
+  extern __shared__ float row[];
+  __shared__ float scratch[16];
+  __shared__ float inv[64];
+  const size_t r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : r;
+  const int len = hidden / groups;
+  float* res = residual + src * hidden;
+  if (y) {
+    const T* yr = y + r * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) row[i] = to_f32(yr[i]);
+    __syncthreads();
+    for (int g0 = 0; g0 < groups; g0 += 64) {
+      const int n = groups - g0 < 64 ? groups - g0 : 64;
+      for (int g = 0; g < n; ++g) {
+        const float ss = part_square_sum(row, g0 + g, len, scratch);
+        if (threadIdx.x == 0) inv[g] = 1.0f / sqrtf(ss / (float)len + eps);
+      }
+      __syncthreads();
+      for (int i = g0 * len + threadIdx.x; i < (g0 + n) * len; i += blockDim.x) {
+        const float v = res[i] + row[i] * inv[i / len - g0] * w_add[i];
+        res[i] = v;
+        row[i] = v;
+      }
+      __syncthreads();
+    }
+  } else if (out) {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) row[i] = res[i];
+    __syncthreads();
+  }
+  if (!out) return;
+  T* dst = out + r * hidden;
+  for (int g0 = 0; g0 < groups; g0 += 64) {
+    const int n = groups - g0 < 64 ? groups - g0 : 64;
+    for (int g = 0; g < n; ++g) {
+      const float ss = part_square_sum(row, g0 + g, len, scratch);
+      if (threadIdx.x == 0) inv[g] = 1.0f / sqrtf(ss / (float)len + eps);
+    }
+    __syncthreads();
+    for (int i = g0 * len + threadIdx.x; i < (g0 + n) * len; i += blockDim.x)
+      dst[i] = from_f32<T>(row[i] * inv[i / len - g0] * w_out[i]);
+    __syncthreads();
+  }
+}
+
+// out = a N(z) + b N(z^2) + c N(z^3) + e over a row, z = x (+ bias), powers element by element, N(u) = u over
+// sqrt(mean(u^2) + eps); coeff = (a, b, c, e) on the device.  A workgroup a row; the row is read twice.
+template <typename T>
+__global__ __launch_bounds__(kRowThreads) void poly_norm_kernel(const T* __restrict__ x, const float* __restrict__ bias,
+                                                               const float* __restrict__ coeff, T* __restrict__ out,
+                                                               int width, float eps) {
+  __shared__ float scratch[16];
+  const size_t r = blockIdx.x;
+  const T* xr = x + r * width;
+  float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float z = to_f32(xr[i]) + (bias ? bias[i] : 0.f);
+    const float z2 = z * z;
+    s2 += z2;
+    s4 += z2 * z2;
+    s6 += z2 * z2 * z2;
+  }
+  s2 = block_sum(s2, scratch);
+  s4 = block_sum(s4, scratch);
+  s6 = block_sum(s6, scratch);
+  const float n = (float)width;
+  const float a = coeff[0] / sqrtf(s2 / n + eps), b = coeff[1] / sqrtf(s4 / n + eps), c = coeff[2] / sqrtf(s6 / n + eps);
+  const float e = coeff[3];
+  T* dst = out + r * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float z = to_f32(xr[i]) + (bias ? bias[i] : 0.f);
+    dst[i] = from_f32<T>(a * z + b * (z * z) + c * (z * z * z) + e);
+  }
+}
+
+// A wavefront a (row, head): out[r, h, :] = o[r, h, :] / sqrt(mean(o[r, h, :]^2) + eps) * w * act(gate[r, h, :]) * scale.
+// w (or null: no weight) has `vdim` elements shared by the heads; gate act: 0 sigmoid(g), 1 g * sigmoid(g).
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, const T* __restrict__ gate,
+                                                            size_t gate_stride, const float* __restrict__ w,
+                                                            T* __restrict__ out, size_t out_stride, int nrows, int heads,
+                                                            int vdim, float eps, int act, float scale) {
+  const int lane = threadIdx.x % kWave;
+  const size_t item = (size_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (item >= (size_t)nrows * heads) return;
+  const size_t r = item / heads;
+  const int h = (int)(item % heads);
+  const float* src = o + (r * heads + h) * vdim;
+  float ss = 0.f;
+  for (int i = lane; i < vdim; i += kWave) ss += src[i] * src[i];
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
+  const T* g = gate + r * gate_stride + (size_t)h * vdim;
+  T* dst = out + r * out_stride + (size_t)h * vdim;
+  for (int i = lane; i < vdim; i += kWave) {
+    const float gv = to_f32(g[i]);
+    const float sg = 1.0f / (1.0f + expf(-gv));
+    dst[i] = from_f32<T>(src[i] * inv * (w ? w[i] : 1.0f) * (act == 1 ? gv * sg : sg) * scale);
+  }
+}
+
+}  // namespace pa
+
+using namespace pa;
+
+extern "C" int pa_group_norm_step(void* stream, int dtype, const void* y, const float* w_add, float* residual,
+                                  const float* w_out, void* out, const int* rows, int nrows, int hidden, int groups,
+                                  float eps) {
+  if (nrows == 0) return 0;
+  PA_REQUIRE(nrows > 0 && hidden > 0 && groups > 0 && hidden % groups == 0,
+             "group_norm_step: bad sizes rows=%d hidden=%d groups=%d (the groups must divide the row)", nrows, hidden, groups);
+  PA_REQUIRE(hidden <= 16384, "group_norm_step: rows of %d elements are more than the 16384 the kernel takes", hidden);
+  PA_REQUIRE(residual && (y || out), "group_norm_step: needs the stream and a branch to add or an output to write");
+  PA_REQUIRE(!y || w_add, "group_norm_step: a branch to add needs its norm's weight");
+  PA_REQUIRE(!out || w_out, "group_norm_step: an output needs its norm's weight");
+  PA_REQUIRE(!(y && rows), "group_norm_step: rows are chosen only where nothing is added");
+  hipStream_t st = (hipStream_t)stream;
+  const size_t lds = (size_t)hidden * sizeof(float);
+  if (dtype == kF32)
+    hipLaunchKernelGGL(group_norm_step_kernel<float>, dim3(nrows), dim3(kRowThreads), lds, st, (const float*)y, w_add, residual,
+                       w_out, (float*)out, rows, hidden, groups, eps);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(group_norm_step_kernel<bf16>, dim3(nrows), dim3(kRowThreads), lds, st, (const bf16*)y, w_add, residual,
+                       w_out, (bf16*)out, rows, hidden, groups, eps);
+  else
+    return pa::fail("group_norm_step: unknown element type code %d", dtype);
+  return check_launch("group_norm_step");
+}
+
+extern "C" int pa_poly_norm(void* stream, int dtype, const void* x, const float* bias, const float* coeff, void* out,
+                            int nrows, int width, float eps) {
+  if (nrows == 0) return 0;
+  PA_REQUIRE(nrows > 0 && width > 0 && x && coeff && out, "poly_norm: bad sizes rows=%d width=%d or a null operand", nrows, width);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == kF32)
+    hipLaunchKernelGGL(poly_norm_kernel<float>, dim3(nrows), dim3(kRowThreads), 0, st, (const float*)x, bias, coeff,
+                       (float*)out, width, eps);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(poly_norm_kernel<bf16>, dim3(nrows), dim3(kRowThreads), 0, st, (const bf16*)x, bias, coeff, (bf16*)out,
+                       width, eps);
+  else
+    return pa::fail("poly_norm: unknown element type code %d", dtype);
+  return check_launch("poly_norm");
+}
+
+extern "C" int pa_head_norm_gate(void* stream, int dtype, const float* o, const void* gate, long gate_stride, const float* w,
+                                 void* out, long out_stride, int nrows, int heads, int vdim, float eps, int act, float scale) {
+  if (nrows == 0) return 0;
+  PA_REQUIRE(nrows > 0 && heads > 0 && vdim > 0 && gate_stride >= (long)heads * vdim && out_stride >= (long)heads * vdim,
+             "head_norm_gate: bad sizes rows=%d heads=%d vdim=%d gate stride=%ld out stride=%ld", nrows, heads, vdim,
+             gate_stride, out_stride);
+  PA_REQUIRE(act == 0 || act == 1, "head_norm_gate: gate activation code %d is not 0 (sigmoid) or 1 (silu)", act);
+  hipStream_t st = (hipStream_t)stream;
+  const long items = (long)nrows * heads;
+  const int blocks = (int)((items + 3) / 4);
+  if (dtype == kF32)
+    hipLaunchKernelGGL(head_norm_gate_kernel<float>, dim3(blocks), dim3(256), 0, st, o, (const float*)gate, (size_t)gate_stride,
+                       w, (float*)out, (size_t)out_stride, nrows, heads, vdim, eps, act, scale);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(head_norm_gate_kernel<bf16>, dim3(blocks), dim3(256), 0, st, o, (const bf16*)gate, (size_t)gate_stride, w,
+                       (bf16*)out, (size_t)out_stride, nrows, heads, vdim, eps, act, scale);
+  else
+    return pa::fail("head_norm_gate: unknown element type code %d", dtype);
+  return check_launch("head_norm_gate");
+}

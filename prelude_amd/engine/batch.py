@@ -50,6 +50,7 @@ class StepBatch:
     max_decode_context: int = 0  # longest context among decode_seqs
     page_size: int = 0
     graph: Optional[object] = None  # set while a step is being captured or replayed from fixed buffers
+    compute_dtype: Optional[torch.dtype] = None   # the engine's element type, for blocks between which only a 32-bit stream travels
 
     @property
     def all_decode(self) -> bool:

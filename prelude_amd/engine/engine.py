@@ -109,7 +109,8 @@ class Engine:
 
     def _set_cache(self, pages: List[int], state_slots: int) -> None:
         specs = [c.spec for c in self.model.cache_slots]
-        self.tables = PageTables(self.page_size, [(n, g.window) for n, g in zip(pages, self.group_specs)], state_slots)
+        self.tables = PageTables(self.page_size, [(n, g.window, int(getattr(g, "keep_first", 0)))
+                                                  for n, g in zip(pages, self.group_specs)], state_slots)
         self.caches = allocate_storage(specs, self._group_of_slot, pages, self.page_size, state_slots, self.dtype,
                                        self.device)
         self.pages_per_group = list(pages)

@@ -59,24 +59,28 @@ class CausalLM:
         for p, _ in self._parts:
             p.bind(self.shared)
 
-        # caches: one per run that does not read another's
+        # caches: one per run that does not read another's; a mixer made of several (``cache_spec()`` a tuple) has one
+        # per member that keeps something, and gets them as a tuple in that order
         self.cache_slots: List[Optional[CacheSlot]] = []
-        self.run_cache: List[Optional[int]] = []   # run index -> index into cache_slots
+        self.run_cache: List[object] = []   # run index -> None | index into cache_slots | tuple of indices
         for i, r in enumerate(spec.order):
             mixer = getattr(self.blocks[r.layer], "mixer", None)
             cs = mixer.cache_spec() if mixer is not None else None
+            several = isinstance(cs, (tuple, list))
+            wanted = list(cs) if several else ([cs] if cs is not None else [])
             if r.reads_cache_of is not None:
                 src = self.run_cache[r.reads_cache_of]
-                if src is None or self.cache_slots[src].spec != cs:
+                have = [] if src is None else [self.cache_slots[j].spec for j in (src if isinstance(src, tuple) else (src,))]
+                if not have or have != wanted:
                     raise PartError(f"run {i} cannot read the cache of run {r.reads_cache_of}: "
-                                    f"it keeps {self.cache_slots[src].spec if src is not None else None}, "
-                                    f"this layer needs {cs}")
+                                    f"it keeps {have or None}, this layer needs {wanted or None}")
                 self.run_cache.append(src)
-            elif cs is None:
+            elif not wanted:
                 self.run_cache.append(None)
             else:
-                self.cache_slots.append(CacheSlot(i, cs))
-                self.run_cache.append(len(self.cache_slots) - 1)
+                first = len(self.cache_slots)
+                self.cache_slots.extend(CacheSlot(i, w) for w in wanted)
+                self.run_cache.append(tuple(range(first, first + len(wanted))) if several else first)
 
     def _make(self, category: str, ps: PartSpec) -> Part:
         p = build_part(category, ps.kind, ps.params)
@@ -118,7 +122,7 @@ class CausalLM:
                     seen.add(ps.weights[local])
                     n = 1
                     for d in req.shape:
-                        n *= int(d)
+                        n *= max(int(d), 1)
                     total += n
         return total
 
@@ -160,16 +164,18 @@ class CausalLM:
         """
         hidden = self.embedding.forward(step.token_ids)
         residual = None
+        step.compute_dtype = self.dtype
         for i, r in enumerate(self.spec.order):
             ci = self.run_cache[i]
-            cache = caches[ci] if ci is not None else None
+            cache = None if ci is None else (tuple(caches[c] for c in ci) if isinstance(ci, tuple) else caches[ci])
             hidden, residual = self.blocks[r.layer].forward(hidden, residual, step, cache,
                                                             write_cache=r.reads_cache_of is None)
         if step.want_rows.shape[0] == 0:
-            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=hidden.device)
+            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
         if self.blocks[self.spec.order[-1].layer].HANDS_ON_STREAM:
             # the last block handed on the stream itself: nothing waits to be added, the norm is of its rows alone
-            normed = self.final_norm.forward_rows(None, residual, step.want_rows, out_dtype=hidden.dtype)
+            normed = self.final_norm.forward_rows(None, residual, step.want_rows,
+                                                  out_dtype=hidden.dtype if hidden is not None else self.dtype)
             return self.head.forward(normed)
         if not self.final_norm.TAKES_SLICE_SUMS:
             from ..ops import kernels as K

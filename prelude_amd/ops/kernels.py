@@ -1563,3 +1563,224 @@ def latent_attention(q: torch.Tensor, cache: torch.Tensor, sink: Optional[torch.
 def linear_clamped_gate(x: torch.Tensor, w, limit: float, alpha: float) -> torch.Tensor:
     """The clamped gated pair of ``clamped_gate`` over x W^T for a weight [2I, K] whose rows alternate gate_j, up_j."""
     return clamped_gate(linear(x, w), limit, alpha)
+
+
+# ---------------------------------------------------------------------------
+# Statistics over parts of a row
+def group_norm_step(residual: torch.Tensor, groups: int, eps: float, y: Optional[torch.Tensor] = None,
+                    w_add: Optional[torch.Tensor] = None, w_out: Optional[torch.Tensor] = None,
+                    out_dtype: Optional[torch.dtype] = None, rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """One step around a 32-bit stream ``residual`` [T, H], with the RMS norm in groups (the row in ``groups`` equal
+    consecutive parts, each over its own sqrt(mean(part^2) + eps)):
+
+    with ``y`` [T, H] and ``w_add``: residual += norm(y) * w_add, in place;
+    with ``w_out``: returns norm(residual) * w_out in ``out_dtype`` (the next branch's input), of the rows ``rows``
+    alone when given (which goes without ``y``)."""
+    _dev(residual, y, w_add, w_out, rows)
+    _f32(residual, "residual")
+    _f32(w_add, "norm weight")
+    _f32(w_out, "norm weight")
+    if residual.dim() != 2 or not residual.is_contiguous():
+        raise NativeError(f"group_norm_step: the stream {tuple(residual.shape)} is not a contiguous [T, H]")
+    m, h = residual.shape
+    if y is not None and (tuple(y.shape) != (m, h) or w_add is None or tuple(w_add.shape) != (h,) or not y.is_contiguous()):
+        raise NativeError(f"group_norm_step: branch {tuple(y.shape)} / weight beside a stream {tuple(residual.shape)}")
+    if w_out is not None and tuple(w_out.shape) != (h,):
+        raise NativeError(f"group_norm_step: weight {tuple(w_out.shape)} for rows of {h}")
+    n, out = m, None
+    if rows is not None:
+        _i32(rows, "rows")
+        n = rows.shape[0]
+    if w_out is not None:
+        dt = out_dtype if out_dtype is not None else (y.dtype if y is not None else torch.float32)
+        if y is not None and dt != y.dtype:
+            raise NativeError(f"group_norm_step: an output of {dt} beside a branch of {y.dtype}")
+        out = torch.empty((n, h), dtype=dt, device=residual.device)
+    code = _CODES[out.dtype] if out is not None else _code(y)
+    check(kernels().pa_group_norm_step(_stream(), code, _ptr(y), _ptr(w_add), _ptr(residual), _ptr(w_out), _ptr(out), _ptr(rows),
+                                       n, h, int(groups), float(eps)))
+    return out
+
+
+def poly_norm(x: torch.Tensor, coeff: torch.Tensor, eps: float, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """a N(z) + b N(z^2) + c N(z^3) + e over rows, z = x (+ bias), powers element by element, N(u) = u over
+    sqrt(mean(u^2) + eps); ``coeff`` float32 (a, b, c, e) on the device."""
+    _dev(x, coeff, bias)
+    _f32(coeff, "coefficients")
+    _f32(bias, "bias")
+    if x.dim() != 2 or not x.is_contiguous() or tuple(coeff.shape) != (4,) or (bias is not None and tuple(bias.shape) != (x.shape[1],)):
+        raise NativeError(f"poly_norm: x {tuple(x.shape)} / coefficients {tuple(coeff.shape)}")
+    out = torch.empty_like(x)
+    check(kernels().pa_poly_norm(_stream(), _code(x), _ptr(x), _ptr(bias), _ptr(coeff), _ptr(out), x.shape[0], x.shape[1], float(eps)))
+    return out
+
+
+HEAD_GATES = {"sigmoid": 0, "silu": 1}
+
+
+def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, weight: Optional[torch.Tensor], eps: float, gate_activation: str = "sigmoid",
+                   out: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
+    """o float32 [T, heads, vdim]: every head over its own sqrt(mean^2 + eps), times ``weight`` (float32 [vdim], shared by
+    the heads; None: none), times act(gate) (``gate`` [T, heads * vdim] of the engine's type, rows may lie inside a
+    wider tensor), times ``scale``.  Written to ``out`` (rows may lie inside a wider tensor) or a fresh [T, heads * vdim]."""
+    _dev(o, weight)
+    _f32(o, "head_norm_gate input")
+    _f32(weight, "norm weight")
+    if o.dim() != 3 or not o.is_contiguous():
+        raise NativeError(f"head_norm_gate: o {tuple(o.shape)} is not a contiguous [T, heads, vdim]")
+    t, heads, vdim = o.shape
+    if gate_activation not in HEAD_GATES:
+        raise NativeError(f"head_norm_gate: gate activation {gate_activation!r} is not one of {sorted(HEAD_GATES)}")
+    if not gate.is_cuda or gate.dim() != 2 or gate.stride(1) != 1 or tuple(gate.shape) != (t, heads * vdim) or \
+            (weight is not None and tuple(weight.shape) != (vdim,)):
+        raise NativeError(f"head_norm_gate: gate {tuple(gate.shape)} / weight for o {tuple(o.shape)}")
+    if out is None:
+        out = torch.empty((t, heads * vdim), dtype=gate.dtype, device=o.device)
+    elif out.dtype != gate.dtype or tuple(out.shape) != (t, heads * vdim) or out.stride(1) != 1:
+        raise NativeError(f"head_norm_gate: out {tuple(out.shape)} {out.dtype}")
+    if t:
+        check(kernels().pa_head_norm_gate(_stream(), _code(gate), _ptr(o), gate.data_ptr(), gate.stride(0), _ptr(weight),
+                                          out.data_ptr(), out.stride(0), t, heads, vdim, float(eps), HEAD_GATES[gate_activation],
+                                          float(scale)))
+    return out
+
+
+# ---------------------------------------------------------------------------
+# Attention with a window that keeps first tokens, a bias by distance and a gate a head
+def qkv_prepare(p: torch.Tensor, q_off: int, k_off: int, v_off: int, q_weight: Optional[torch.Tensor],
+                k_weight: Optional[torch.Tensor], slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
+                v_cache: Optional[torch.Tensor], nh: int, nkv: int, hd: int, vd: int, eps: float) -> torch.Tensor:
+    """From the merged projection ``p`` [T, width] (rows may lie inside a wider tensor): the queries [T, nh, hd], with
+    ``q_weight`` (float32 [nh * hd]) brought to unit RMS over the whole projection and multiplied by it; keys (the
+    same with ``k_weight``) and values written to the caches at ``slots`` (None: queries only)."""
+    _dev(p, q_weight, k_weight, slots, k_cache, v_cache)
+    _f32(q_weight, "query norm weight")
+    _f32(k_weight, "key norm weight")
+    if p.dim() != 2 or p.stride(1) != 1:
+        raise NativeError(f"qkv_prepare: projection {tuple(p.shape)} with strides {p.stride()}")
+    t = p.shape[0]
+    if (q_weight is not None and tuple(q_weight.shape) != (nh * hd,)) or (k_weight is not None and tuple(k_weight.shape) != (nkv * hd,)):
+        raise NativeError("qkv_prepare: a norm weight does not have its projection's size")
+    page = 0
+    if slots is not None:
+        _i32(slots, "slots")
+        if slots.shape != (t,) or k_cache is None or v_cache is None or k_cache.dtype != p.dtype or v_cache.dtype != p.dtype or \
+                tuple(k_cache.shape[1:]) != (nkv, k_cache.shape[2], hd) or tuple(v_cache.shape) != (k_cache.shape[0], nkv, vd, k_cache.shape[2]):
+            raise NativeError(f"qkv_prepare: caches {None if k_cache is None else tuple(k_cache.shape)} / "
+                              f"{None if v_cache is None else tuple(v_cache.shape)} for {nkv} heads of {hd} and {vd}")
+        page = k_cache.shape[2]
+    q = torch.empty((t, nh, hd), dtype=p.dtype, device=p.device)
+    if t:
+        check(kernels().pa_qkv_prepare(_stream(), _code(p), p.data_ptr(), p.stride(0), int(q_off), int(k_off), int(v_off),
+                                       _ptr(q_weight), _ptr(k_weight), _ptr(slots), _ptr(q), _ptr(k_cache) if slots is not None else None,
+                                       _ptr(v_cache) if slots is not None else None, t, nh, nkv, hd, vd, page, float(eps)))
+    return q
+
+
+def attention_masked(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, group, step, window: int, keep_first: int,
+                     scale: float, softcap: float = 0.0, slopes: Optional[torch.Tensor] = None,
+                     sink: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                     out: Optional[torch.Tensor] = None, out_scale: float = 1.0) -> torch.Tensor:
+    """Paged causal attention of one step over one cache group, any mix of portions and single tokens.  The query at
+    i sees the key at j <= i when i - j < ``window`` (0: no window) or j < ``keep_first``.  score = q.k * scale, bent
+    to cap * tanh(score / cap) for ``softcap`` > 0, less ``slopes``[h] * (i - j); ``sink`` [heads] joins the softmax's
+    denominator; ``gate`` [T, heads] (rows may lie inside a wider tensor): a head's output times sigmoid(gate), and
+    ``out_scale``, before rounding.  q [T, nh, hd]; K cache [pages, nkv, page, hd]; V cache [pages, nkv, vd, page].
+    Returns (or fills ``out``, whose rows may lie inside a wider tensor) [T, nh * vd]."""
+    _dev(q, k_cache, v_cache, slopes, sink)
+    if q.dim() != 3 or not q.is_contiguous() or k_cache.dim() != 4 or v_cache.dim() != 4:
+        raise NativeError(f"attention_masked: q {tuple(q.shape)} / caches")
+    t, nh, hd = q.shape
+    pages, nkv, page, khd = k_cache.shape
+    vd = v_cache.shape[2]
+    if khd != hd or tuple(v_cache.shape) != (pages, nkv, vd, page) or k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
+        raise NativeError(f"attention_masked: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} for q {tuple(q.shape)} {q.dtype}")
+    for name, v in (("slopes", slopes), ("sink", sink)):
+        if v is not None:
+            _f32(v, name)
+            if tuple(v.shape) != (nh,):
+                raise NativeError(f"attention_masked: {name} {tuple(v.shape)} for {nh} heads")
+    if gate is not None and (not gate.is_cuda or gate.dtype != q.dtype or gate.dim() != 2 or tuple(gate.shape) != (t, nh) or gate.stride(1) != 1):
+        raise NativeError(f"attention_masked: gate {tuple(gate.shape)} {gate.dtype} for {t} tokens of {nh} heads")
+    if out is None:
+        out = torch.empty((t, nh * vd), dtype=q.dtype, device=q.device)
+    elif out.dtype != q.dtype or tuple(out.shape) != (t, nh * vd) or out.stride(1) != 1:
+        raise NativeError(f"attention_masked: out {tuple(out.shape)} {out.dtype}")
+    if t:
+        check(kernels().pa_attn_masked(_stream(), _code(q), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(group.block_table),
+                                       group.block_table.shape[1], _ptr(step.seq_of_token), _ptr(step.positions), out.data_ptr(),
+                                       out.stride(0), t, nh, nkv, hd, vd, page, int(window), int(keep_first), float(scale),
+                                       float(softcap), _ptr(slopes), _ptr(sink), gate.data_ptr() if gate is not None else None,
+                                       gate.stride(0) if gate is not None else 0, float(out_scale)))
+    return out
+
+
+# ---------------------------------------------------------------------------
+# The gated delta rule; rotation in front of a recurrence
+def delta_prepare(p: torch.Tensor, off: int, b_off: int, conv_weight: torch.Tensor, conv_state: torch.Tensor, a: torch.Tensor,
+                  a_off: int, a_log: torch.Tensor, dt_bias: torch.Tensor, step, heads: int, kvh: int, d: int, e: int):
+    """What stands in front of the gated delta rule.  ``p`` [T, width] holds from column ``off`` the channels
+    [q | k | v] (q, k: ``kvh`` heads of ``d``; v: ``heads`` heads of ``e``) and at ``b_off`` one gate input a head.
+    Every channel passes a causal convolution (``conv_weight`` float32 [channels, taps], the last tap the token's
+    own; the inputs before the step come from ``conv_state`` float32 [slots, channels, taps - 1], which then moves
+    on) and SiLU; q and k become unit vectors per head, q also times d^(-1/2).  Returns 32-bit
+    (x [T, channels], decay [T, heads, d] = exp(-exp(a_log_h) softplus(a + dt_bias)) from ``a`` [T, .] at column
+    ``a_off``, beta [T, heads] = sigmoid of the gate input)."""
+    _dev(p, conv_weight, conv_state, a, a_log, dt_bias)
+    for name, v in (("convolution weight", conv_weight), ("convolution state", conv_state), ("A_log", a_log), ("dt_bias", dt_bias)):
+        _f32(v, name)
+    t = p.shape[0]
+    c = 2 * kvh * d + heads * e
+    taps = conv_weight.shape[1] if conv_weight.dim() == 2 else 0
+    if p.dim() != 2 or p.stride(1) != 1 or a.dim() != 2 or a.stride(1) != 1 or a.dtype != p.dtype or a.shape[0] != t or \
+            tuple(conv_weight.shape) != (c, taps) or conv_state.dim() != 3 or tuple(conv_state.shape[1:]) != (c, max(taps - 1, 0)) or \
+            tuple(a_log.shape) != (heads,) or tuple(dt_bias.shape) != (heads * d,) or not conv_state.is_contiguous():
+        raise NativeError(f"delta_prepare: p {tuple(p.shape)} / conv {tuple(conv_weight.shape)} / state {tuple(conv_state.shape)} / "
+                          f"a {tuple(a.shape)} for {heads} heads ({kvh} of keys) of {d} and {e}")
+    x = torch.empty((t, c), dtype=torch.float32, device=p.device)
+    decay = torch.empty((t, heads, d), dtype=torch.float32, device=p.device)
+    beta = torch.empty((t, heads), dtype=torch.float32, device=p.device)
+    if t:
+        check(kernels().pa_delta_prepare(_stream(), _code(p), p.data_ptr(), p.stride(0), int(off), int(b_off), _ptr(conv_weight), taps,
+                                         _ptr(conv_state), _ptr(step.seq_of_token), _ptr(step.cu_q), _ptr(step.state_slots),
+                                         a.data_ptr(), a.stride(0), int(a_off), _ptr(a_log), _ptr(dt_bias), _ptr(x), _ptr(decay),
+                                         _ptr(beta), t, step.num_seqs, heads, kvh, d, e))
+    return x, decay, beta
+
+
+def gated_delta(x: torch.Tensor, decay: torch.Tensor, beta: torch.Tensor, state: torch.Tensor, step, heads: int, kvh: int,
+                d: int, e: int) -> torch.Tensor:
+    """The gated delta rule over the step's sequences, token by token: per head S <- diag(g) S; u = beta (v - S^T k);
+    S <- S + k u^T; o = S^T q.  ``x``, ``decay``, ``beta`` as ``delta_prepare`` returns them; ``state`` float32
+    [slots, heads, d, e], read and left through ``step.state_slots``.  Returns float32 [T, heads, e]."""
+    _dev(x, decay, beta, state)
+    for name, v in (("x", x), ("decay", decay), ("beta", beta), ("state", state)):
+        _f32(v, name)
+    t = x.shape[0]
+    if tuple(x.shape) != (t, 2 * kvh * d + heads * e) or tuple(decay.shape) != (t, heads, d) or tuple(beta.shape) != (t, heads) or \
+            state.dim() != 4 or tuple(state.shape[1:]) != (heads, d, e) or not state.is_contiguous():
+        raise NativeError(f"gated_delta: x {tuple(x.shape)} / decay {tuple(decay.shape)} / beta {tuple(beta.shape)} / state {tuple(state.shape)}")
+    out = torch.empty((t, heads, e), dtype=torch.float32, device=x.device)
+    if t:
+        check(kernels().pa_gated_delta(_stream(), _ptr(x), _ptr(decay), _ptr(beta), _ptr(state), _ptr(step.state_slots), _ptr(step.cu_q),
+                                       _ptr(out), step.num_seqs, heads, kvh, d, e))
+    return out
+
+
+def rotate_halves_f32(p: torch.Tensor, q_off: int, k_off: int, v_off: int, inv_freq: Optional[torch.Tensor],
+                      positions: torch.Tensor, heads: int, d: int, e: int, rot: int, k_scale: float = 1.0) -> torch.Tensor:
+    """From ``p`` [T, width]: queries and keys (``heads`` heads of ``d`` from ``q_off`` and ``k_off``) with the first
+    ``rot`` dimensions of every head turned, dimension i with i + rot / 2, by position * inv_freq[i], the keys then times
+    ``k_scale``; values (``heads`` heads of ``e`` from ``v_off``) as they are.  All in 32-bit:
+    returns float32 [T, 2 * heads * d + heads * e] = [q | k | v]."""
+    _dev(p, inv_freq, positions)
+    _f32(inv_freq, "rotary frequencies")
+    _i32(positions, "positions")
+    t = p.shape[0]
+    if p.dim() != 2 or p.stride(1) != 1 or positions.shape != (t,) or (rot and (inv_freq is None or tuple(inv_freq.shape) != (rot // 2,))):
+        raise NativeError(f"rotate_halves: p {tuple(p.shape)} / positions / frequencies for {rot} turned dimensions")
+    out = torch.empty((t, 2 * heads * d + heads * e), dtype=torch.float32, device=p.device)
+    if t:
+        check(kernels().pa_rotate_halves_f32(_stream(), _code(p), p.data_ptr(), p.stride(0), int(q_off), int(k_off), int(v_off),
+                                             _ptr(inv_freq), _ptr(positions), _ptr(out), t, heads, d, e, int(rot), float(k_scale)))
+    return out

@@ -11,6 +11,7 @@ projection (qwen3.rs:226-228).
 """
 from __future__ import annotations
 
+import dataclasses
 import math
 from typing import Optional
 
@@ -142,3 +143,130 @@ class GQAAttention(Mixer):
                                  self.rotary_dim, self.norm_eps, **({"inv_freq": freq} if freq is not None else {}))
         o = K.attention(q, cache.k, cache.v, g, step, self.window, self.scale, self.score_cap, sink=self.sinks)
         return K.linear(o.view(o.shape[0], nh * hd), self.w_o, self.b_o, slices_ok=True)
+
+
+@dataclasses.dataclass(frozen=True)
+class KeptFirstKVCacheSpec(KVCacheSpec):
+    """Keys and values in pages under a window that keeps the first tokens: pages that hold one of the first
+    ``keep_first`` positions are never given back while the request lives."""
+    keep_first: int = 0
+
+
+@register_part("mixer", "windowed_attention")
+class WindowedAttention(Mixer):
+    """Grouped-query attention without rotation whose mask is a window that keeps the first tokens: the query at i
+    sees the key at j <= i when i - j < ``window`` (0: no window) or j < ``keep_first``.  Values have a width of their
+    own.  Optional, each a parameter: queries and keys brought to unit RMS over the whole projection (all heads at once)
+    times a weight of that size (``qk_norm="whole"``); scores bent to cap * tanh(score / cap) (``score_cap``); a bias by
+    distance, slope_h (i - j) taken off the score with slope_h = 2^(-``slope_exponent`` (h + 1) / heads)
+    (``slope_exponent`` > 0); a learned sink per head in the softmax's denominator (``sink="learned"``); a gate per
+    head, the head's output times sigmoid(W_g x)_h (``head_gate``).
+
+    ``cache_window`` / ``cache_keep_first``: the mask the cache is kept for, where it is wider than this layer's own
+    because other layers read the same keys (``window`` 0 = everything)."""
+    LAUNCHES = 4   # merged projection, norm + cache write, attention, output projection
+    GRAPH_SAFE_PORTIONS = True
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, scale: float,
+                 window: int = 0, keep_first: int = 0, qk_norm: Optional[str] = None, norm_eps: float = 1e-6,
+                 score_cap: float = 0.0, slope_exponent: float = 0.0, sink: Optional[str] = None, head_gate: bool = False,
+                 own_keys: bool = True, cache_window: Optional[int] = None, cache_keep_first: Optional[int] = None):
+        if num_heads % num_kv_heads:
+            raise PartError(f"windowed_attention: {num_heads} heads are not a multiple of {num_kv_heads} KV heads")
+        if not (1 <= head_dim <= 256 and 1 <= value_dim <= 256):
+            raise PartError(f"windowed_attention: key width {head_dim} or value width {value_dim} is outside 1..256")
+        if qk_norm not in (None, "whole"):
+            raise PartError(f"windowed_attention: qk_norm {qk_norm!r} is not one of None, 'whole'")
+        if sink not in (None, "learned"):
+            raise PartError(f"windowed_attention: sink {sink!r} is not one of None, 'learned'")
+        if window < 0 or keep_first < 0 or score_cap < 0 or slope_exponent < 0:
+            raise PartError("windowed_attention: window, kept first tokens, score cap and slope exponent must not be negative")
+        self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.head_dim, self.value_dim, self.scale = int(head_dim), int(value_dim), float(scale)
+        self.window, self.keep_first = int(window), int(keep_first) if window else 0
+        self.qk_norm, self.norm_eps, self.score_cap = qk_norm, float(norm_eps), float(score_cap)
+        self.slope_exponent, self.sink, self.head_gate = float(slope_exponent), sink, bool(head_gate)
+        # False: this layer has no key and value projections and reads the keys and values another layer cached
+        self.own_keys = bool(own_keys)
+        self.cache_window = self.window if cache_window is None else int(cache_window)
+        self.cache_keep_first = self.keep_first if cache_keep_first is None else int(cache_keep_first)
+        if self.cache_window and (not self.window or self.cache_window < self.window or
+                                  self.cache_keep_first < self.keep_first):
+            raise PartError("windowed_attention: the cache's mask must hold everything this layer's mask sees")
+        self.w_in = self.w_o = self.q_norm = self.k_norm = self.sinks = self.slopes = None
+
+    # ---- sizes of its columns in the projection of its input ----
+    @property
+    def nq(self) -> int:
+        return self.num_heads * self.head_dim
+
+    @property
+    def nk(self) -> int:
+        return self.num_kv_heads * self.head_dim if self.own_keys else 0
+
+    @property
+    def nv(self) -> int:
+        return self.num_kv_heads * self.value_dim if self.own_keys else 0
+
+    @property
+    def mixed_size(self) -> int:
+        """Width of what ``mix`` leaves for the output projection."""
+        return self.num_heads * self.value_dim
+
+    def cache_spec(self):
+        if self.cache_window and self.cache_keep_first:
+            return KeptFirstKVCacheSpec(self.num_kv_heads, self.head_dim, self.cache_window, self.value_dim, self.cache_keep_first)
+        return KVCacheSpec(self.num_kv_heads, self.head_dim, self.cache_window, self.value_dim)
+
+    def tensors(self):
+        h = self.hidden_size
+        t = {"q": TensorReq((self.nq, h), MATRIX), "o": TensorReq((h, self.mixed_size), MATRIX)}
+        if self.own_keys:
+            t.update({"k": TensorReq((self.nk, h), MATRIX), "v": TensorReq((self.nv, h), MATRIX)})
+        if self.qk_norm:
+            t["q.norm"] = TensorReq((self.nq,), NORM)
+            if self.own_keys:
+                t["k.norm"] = TensorReq((self.nk,), NORM)
+        if self.sink:
+            t["sink"] = TensorReq((self.num_heads,), VECTOR)
+        if self.head_gate:
+            t["g"] = TensorReq((self.num_heads, h), MATRIX)
+        return t
+
+    def input_rows(self, tensors) -> torch.Tensor:
+        """The rows of the product of its input this mixer wants, [q | k | v | gate]; keeps its other tensors."""
+        rows = [tensors["q"]] + ([tensors["k"], tensors["v"]] if self.own_keys else []) + ([tensors["g"]] if self.head_gate else [])
+        if self.qk_norm:
+            self.q_norm = tensors["q.norm"]
+            self.k_norm = tensors["k.norm"] if self.own_keys else None
+        self.sinks = tensors["sink"] if self.sink else None
+        if self.slope_exponent:
+            nh = self.num_heads
+            self.slopes = torch.tensor([2.0 ** (-self.slope_exponent * (i + 1) / nh) for i in range(nh)], dtype=torch.float64) \
+                .to(torch.float32).to(tensors["q"].device)
+        return torch.cat(rows, dim=0) if len(rows) > 1 else rows[0]
+
+    def load(self, tensors, dtype, device):
+        self.w_in = K.prepare_weight(self.input_rows(tensors).contiguous())
+        self.w_o = K.prepare_weight(tensors["o"])
+
+    def mix(self, x, p, off, step, cache, write_cache, out=None, out_scale=1.0):
+        """From the product ``p`` of its input ``x`` (its columns start at ``off``) to the heads' outputs side by side
+        [T, heads * value_dim], times ``out_scale``, into ``out`` when given."""
+        if write_cache != self.own_keys:
+            raise PartError("windowed_attention: a layer with key and value projections writes its own cache, one without "
+                            "reads another's")
+        nh, nkv, hd, vd = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
+        g = step.kv[cache.group]
+        q = K.qkv_prepare(p, off, off + self.nq, off + self.nq + self.nk, self.q_norm, self.k_norm,
+                          g.slots if write_cache else None, cache.k, cache.v, nh, nkv, hd, vd, self.norm_eps)
+        gate = p[:, off + self.nq + self.nk + self.nv: off + self.nq + self.nk + self.nv + nh] if self.head_gate else None
+        if not self.keep_first and self.slopes is None and gate is None and vd == hd and out is None and out_scale == 1.0:
+            o = K.attention(q, cache.k, cache.v, g, step, self.window, self.scale, self.score_cap, sink=self.sinks)
+            return o.view(o.shape[0], nh * vd)
+        return K.attention_masked(q, cache.k, cache.v, g, step, self.window, self.keep_first, self.scale, self.score_cap,
+                                  self.slopes, self.sinks, gate, out, out_scale)
+
+    def forward(self, x, step, cache, write_cache=True):
+        p = K.linear(x, self.w_in)
+        return K.linear(self.mix(x, p, 0, step, cache, write_cache), self.w_o, slices_ok=True)

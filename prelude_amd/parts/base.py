@@ -8,7 +8,8 @@ tensors it needs (by local name and shape), receives them, and runs.
 Categories and the interface each must have:
 
 ``norm``      ``forward(x)``, ``forward_residual(x, residual) -> (residual, normed)``,
-              ``forward_rows(x, residual, rows)``; for blocks that norm a branch's output, ``forward_branch``; ``as_rms() -> (gain, eps) | None`` (given by the base class:
+              ``forward_rows(x, residual, rows)``; for blocks that norm a branch's output, ``forward_branch``; for blocks
+              with a norm in front of and behind every branch also ``forward_stream`` and ``forward_branch_then``; ``as_rms() -> (gain, eps) | None`` (given by the base class:
               None) tells a kernel behind it that it may do the plain RMS formula itself
 ``mixer``/``ffn`` may return their last product as ``ops.kernels.SliceSums`` (``linear(..., slices_ok=True)``):
               only a norm reads it, and one that says ``TAKES_SLICE_SUMS`` adds the slices itself
@@ -43,7 +44,7 @@ TABLE = "table"     # int32; every row distinct integers below ``TensorReq.high`
 
 @dataclasses.dataclass(frozen=True)
 class TensorReq:
-    shape: Tuple[int, ...]
+    shape: Tuple[int, ...]   # a size of -1: whatever the stored tensor has
     kind: str = MATRIX
     high: int = 0       # TABLE: entries are integers in [0, high)
 
@@ -59,6 +60,7 @@ class PagedCacheSpec:
     """
     PAGED = True
     window: int = 0
+    keep_first: int = 0    # with a window: the first positions every later token still sees; their pages are never given back
 
     def bytes_per_token(self, element_size: int) -> int:
         """Bytes a token takes in this mixer's storage, for an engine element of ``element_size`` bytes."""
@@ -282,6 +284,17 @@ class Norm(Part):
         that is to be the final norm behind such a block also takes ``forward_rows(None, residual, rows,
         out_dtype=)``: the norm of the stream's rows alone."""
         raise NotImplementedError
+
+    def forward_stream(self, residual: torch.Tensor, out_dtype):
+        """The norm of every row of a 32-bit stream, in ``out_dtype``: a branch's input where the norm sits in front of
+        the branch and nothing waits to be added."""
+        raise NotImplementedError
+
+    def forward_branch_then(self, y, residual: torch.Tensor, then: Optional["Norm"], out_dtype):
+        """residual += norm(y) as ``forward_branch``, then the next branch's input ``then.forward_stream(residual)``
+        (None when ``then`` is None).  A norm that can do both in one launch does so; this is the plain order."""
+        self.forward_branch(y, residual, None)
+        return then.forward_stream(residual, out_dtype) if then is not None else None
 
 
 class PositionEncoding(Part):

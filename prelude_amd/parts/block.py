@@ -14,7 +14,7 @@ from __future__ import annotations
 import torch
 
 from ..ops import kernels as K
-from .base import Block, register_part
+from .base import Block, PartError, register_part
 
 
 @register_part("block", "prenorm")
@@ -106,3 +106,61 @@ class BranchNormMixerBlock(Block):
         hidden, residual = BranchNormBlock._enter(hidden, residual)
         y = self.mixer.forward(hidden, step, cache, write_cache)
         return BranchNormBlock._add(self.mixer_norm, y, hidden, residual), residual
+
+
+@register_part("block", "sandwich_norm")
+class SandwichNormBlock(Block):
+    """A norm in front of and behind every branch: x <- x + post_mixer_norm(mixer(pre_mixer_norm(x))), then
+    x <- x + post_ffn_norm(ffn(pre_ffn_norm(x))).  The stream x is 32-bit and is all that travels between such blocks
+    (``hidden`` is handed on as None); the add behind the mixer and the norm in front of the feed-forward are one
+    launch where the norms can."""
+    GRAPH_SAFE_PORTIONS = True
+    HANDS_ON_STREAM = True
+
+    SLOTS = {"pre_mixer_norm": "norm", "mixer": "mixer", "post_mixer_norm": "norm", "pre_ffn_norm": "norm", "ffn": "ffn",
+             "post_ffn_norm": "norm"}
+
+    def __init__(self, pre_mixer_norm, mixer, post_mixer_norm, pre_ffn_norm, ffn, post_ffn_norm):
+        self.pre_mixer_norm, self.mixer, self.post_mixer_norm = pre_mixer_norm, mixer, post_mixer_norm
+        self.pre_ffn_norm, self.ffn, self.post_ffn_norm = pre_ffn_norm, ffn, post_ffn_norm
+
+    @staticmethod
+    def _enter(hidden, residual, step):
+        """(the stream, the engine's element type: ``step.compute_dtype``).  The first block turns the embedding into
+        the stream."""
+        if residual is None:
+            hidden = K.as_tensor(hidden)
+            return (hidden if hidden.dtype == torch.float32 else K.to_f32(hidden)), hidden.dtype
+        if residual.dtype != torch.float32:
+            raise PartError("sandwich_norm: the stream between such blocks is 32-bit")
+        if hidden is None and step.compute_dtype is None:
+            raise PartError("sandwich_norm: the step does not say the engine's element type")
+        return residual, (hidden.dtype if hidden is not None else step.compute_dtype)
+
+    def forward(self, hidden, residual, step, cache, write_cache=True):
+        residual, dtype = self._enter(hidden, residual, step)
+        h = self.pre_mixer_norm.forward_stream(residual, dtype)
+        y = self.mixer.forward(h, step, cache, write_cache)
+        h = self.post_mixer_norm.forward_branch_then(y, residual, self.pre_ffn_norm, dtype)
+        y = self.ffn.forward(h, step=step) if getattr(self.ffn, "NEEDS_STEP", False) else self.ffn.forward(h)
+        self.post_ffn_norm.forward_branch_then(y, residual, None, dtype)
+        return None, residual
+
+
+@register_part("block", "sandwich_norm_mixer_only")
+class SandwichNormMixerBlock(Block):
+    """A ``sandwich_norm`` layer without a feed-forward: x <- x + post_mixer_norm(mixer(pre_mixer_norm(x)))."""
+    GRAPH_SAFE_PORTIONS = True
+    HANDS_ON_STREAM = True
+
+    SLOTS = {"pre_mixer_norm": "norm", "mixer": "mixer", "post_mixer_norm": "norm"}
+
+    def __init__(self, pre_mixer_norm, mixer, post_mixer_norm):
+        self.pre_mixer_norm, self.mixer, self.post_mixer_norm = pre_mixer_norm, mixer, post_mixer_norm
+
+    def forward(self, hidden, residual, step, cache, write_cache=True):
+        residual, dtype = SandwichNormBlock._enter(hidden, residual, step)
+        h = self.pre_mixer_norm.forward_stream(residual, dtype)
+        y = self.mixer.forward(h, step, cache, write_cache)
+        self.post_mixer_norm.forward_branch_then(y, residual, None, dtype)
+        return None, residual

@@ -15,7 +15,7 @@ from __future__ import annotations
 import torch
 
 from ..ops import kernels as K
-from .base import MATRIX, FeedForward, PartError, TensorReq, register_part
+from .base import MATRIX, VECTOR, FeedForward, PartError, TensorReq, register_part
 
 
 @register_part("ffn", "gated_mlp")
@@ -102,3 +102,29 @@ class SquaredReluMLP(FeedForward):
 
     def forward(self, x):
         return K.linear(K.relu_squared(K.linear(x, self.up)), self.down, slices_ok=True)
+
+
+@register_part("ffn", "poly_norm_mlp")
+class PolyNormMLP(FeedForward):
+    """down(act(up(x))) with biases on both products and act(z) = a N(z) + b N(z^2) + c N(z^3) + e: powers element by
+    element, N(u) = u over sqrt(mean(u^2) + eps) across the inner size, (a, b, c, e) four learned numbers.  The first
+    product's bias is added where the activation reads z."""
+    LAUNCHES = 3
+    GRAPH_SAFE_PORTIONS = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, eps: float):
+        self.hidden_size, self.intermediate_size, self.eps = int(hidden_size), int(intermediate_size), float(eps)
+        self.up = self.down = self.up_bias = self.down_bias = self.coeff = None
+
+    def tensors(self):
+        h, i = self.hidden_size, self.intermediate_size
+        return {"up": TensorReq((i, h), MATRIX), "up.b": TensorReq((i,), VECTOR), "down": TensorReq((h, i), MATRIX),
+                "down.b": TensorReq((h,), VECTOR), "act": TensorReq((4,), VECTOR)}
+
+    def load(self, tensors, dtype, device):
+        self.up, self.down = K.prepare_weight(tensors["up"]), K.prepare_weight(tensors["down"])
+        self.up_bias, self.down_bias, self.coeff = tensors["up.b"], tensors["down.b"], tensors["act"]
+
+    def forward(self, x):
+        z = K.linear(x, self.up)
+        return K.linear(K.poly_norm(z, self.coeff, self.eps, bias=self.up_bias), self.down, self.down_bias)

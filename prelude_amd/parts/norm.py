@@ -77,3 +77,55 @@ class RMSNorm(Norm):
         if residual.dtype != torch.float32:
             raise PartError("rms_norm: a branch is normed and added to a 32-bit stream only")
         return K.rmsnorm_branch(y, self.weight, self.eps, residual, copy_dtype)
+
+
+@register_part("norm", "group_rms_norm")
+class GroupRMSNorm(Norm):
+    """RMS norm in groups around a 32-bit stream: the row is split into ``groups`` equal consecutive parts, each is
+    divided by its own sqrt(mean(part^2) + eps), and the whole is multiplied by the weight.  One group is the plain
+    RMS norm.  It norms the stream for a branch (``forward_stream``), norms a branch's output and adds it to the
+    stream (``forward_branch``), or both in one launch (``forward_branch_then``: the add, then the next branch's
+    input through another norm of this kind)."""
+    GRAPH_SAFE_PORTIONS = True
+
+    def __init__(self, size: int, eps: float, groups: int = 1):
+        self.size, self.eps, self.groups = int(size), float(eps), int(groups)
+        if self.groups < 1 or self.size % self.groups:
+            raise PartError(f"group_rms_norm: {groups} groups do not divide a row of {size}")
+        self.weight: Optional[torch.Tensor] = None
+
+    def tensors(self):
+        return {"weight": TensorReq((self.size,), NORM)}
+
+    def load(self, tensors, dtype, device):
+        self.weight = tensors["weight"]
+
+    def as_rms(self):
+        return (self.weight, self.eps) if self.groups == 1 else None
+
+    @staticmethod
+    def _stream(residual):
+        if residual is None or residual.dtype != torch.float32:
+            raise PartError("group_rms_norm: works around a 32-bit stream")
+        return residual
+
+    def forward_stream(self, residual, out_dtype):
+        return K.group_norm_step(self._stream(residual), self.groups, self.eps, w_out=self.weight, out_dtype=out_dtype)
+
+    def forward_rows(self, x, residual, rows, out_dtype=None):
+        if x is not None:
+            raise PartError("group_rms_norm: nothing waits to be added to the stream when its rows are normed")
+        return K.group_norm_step(self._stream(residual), self.groups, self.eps, w_out=self.weight,
+                                 out_dtype=out_dtype or torch.float32, rows=rows)
+
+    def forward_branch(self, y, residual, copy_dtype=None):
+        if copy_dtype not in (None, torch.float32):
+            raise PartError("group_rms_norm: the stream has no rounded copy; ask `forward_branch_then` for the next branch's input")
+        K.group_norm_step(self._stream(residual), self.groups, self.eps, y=K.as_tensor(y), w_add=self.weight)
+        return None
+
+    def forward_branch_then(self, y, residual, then, out_dtype):
+        if isinstance(then, GroupRMSNorm) and then.groups == self.groups and then.eps == self.eps:
+            return K.group_norm_step(self._stream(residual), self.groups, self.eps, y=K.as_tensor(y), w_add=self.weight,
+                                     w_out=then.weight, out_dtype=out_dtype)
+        return super().forward_branch_then(y, residual, then, out_dtype)

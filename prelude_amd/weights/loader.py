@@ -39,7 +39,8 @@ def check_tensors(requests: Mapping[str, TensorReq], files: WeightFiles, where: 
             missing.append(name)
             continue
         dt, shape = files.info(name)
-        if tuple(shape) != tuple(req.shape):
+        # a size of -1 is left to the tensor (the part that asked checks what it gets against its other tensors)
+        if len(shape) != len(req.shape) or any(want not in (-1, int(got)) for want, got in zip(req.shape, shape)):
             wrong.append(f"{name}: expected {list(req.shape)}, got {list(shape)}")
         elif not (dt.is_floating_point or dt in (torch.int32, torch.int64)):
             wrong.append(f"{name}: element type {dt} cannot be used")

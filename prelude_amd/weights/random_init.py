@@ -69,6 +69,9 @@ def _standard_normal(n: int, key: int, device: torch.device) -> torch.Tensor:
 
 
 def _draw(name: str, req, seed: int, std: float, norm_std: float, device: torch.device) -> torch.Tensor:
+    if any(int(d) < 0 for d in req.shape):
+        raise ValueError(f"tensor {name!r} has a size {list(req.shape)} that only a stored tensor settles; to draw weights, "
+                         f"the configuration has to give it")
     n = 1
     for d in req.shape:
         n *= int(d)
