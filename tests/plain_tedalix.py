@@ -280,3 +280,60 @@ def random_weights(config, seed, dtype=torch.bfloat16):
             t = torch.randn(shape, generator=g) / math.sqrt(shape[-1])
         out[name] = t.to(dtype)
     return out
+
+
+# ---- configurations of the tests' own --------------------------------------------------------------------------------
+def _dense(ff):
+    return {"kind": "dense", "ff": ff}
+
+
+def tiny_config_p():
+    """Three norm groups; a parallel layer whose delta rule shares key heads and has four taps; windowed attention with
+    kept first tokens and values narrower than keys; a retention layer without feed-forward, half of a head turned, a
+    decay of 1; a layer that reads the second layer's keys under a wider mask of its own; a mixer-only last layer."""
+    return {"architecture": "Tedalix", "vocab": 96, "width": 48, "norm": {"eps": 1e-5, "groups": 3}, "layers": [
+        {"type": "parallel", "mlp": _dense(80), "mixer": {
+            "left": {"heads": 3, "kv_heads": 1, "dim": 16, "vdim": 24, "scale": 0.2, "softcap": 15.0, "mask": {"size": 20}},
+            "right": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 24, "conv": 4, "rank": 8},
+            "left_scale": 0.7, "right_scale": 1.1}},
+        {"type": "attention", "mlp": _dense(64), "mixer": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 8, "scale": 0.25,
+                                                          "mask": {"size": 24, "keep_first": 5}}},
+        {"type": "retention", "mlp": None, "mixer": {"heads": 3, "dim": 16, "vdim": 8, "decay": [0.9, 0.99, 1.0],
+                                                     "rot": {"base": 10000.0, "dims": 8}}},
+        {"type": "attention", "mlp": _dense(64), "mixer": {"heads": 2, "kv_heads": 2, "dim": 16, "vdim": 8, "scale": 0.3,
+                                                          "kv_from": 1, "mask": {"size": 40, "keep_first": 2}}},
+        {"type": "retention", "mlp": None, "mixer": {"heads": 2, "dim": 8, "vdim": 24, "decay": [0.5, 0.97],
+                                                     "rot": {"base": 500.0, "dims": 8}}},
+    ]}
+
+
+def tiny_config_q():
+    """One norm group; attention under a plain window (no kept tokens) with keys and values of 64, attention that sees
+    everything, a retention layer without rotation, a parallel layer of one head each without a score cap, two taps."""
+    return {"architecture": "Tedalix", "vocab": 128, "width": 64, "norm": {"eps": 1e-6, "groups": 1}, "layers": [
+        {"type": "attention", "mlp": _dense(96), "mixer": {"heads": 2, "kv_heads": 1, "dim": 64, "vdim": 64, "scale": 0.125,
+                                                          "mask": {"size": 33}}},
+        {"type": "retention", "mlp": _dense(32), "mixer": {"heads": 1, "dim": 32, "vdim": 32, "decay": [0.98]}},
+        {"type": "parallel", "mlp": None, "mixer": {
+            "left": {"heads": 1, "kv_heads": 1, "dim": 32, "vdim": 16, "scale": 0.18, "mask": {"size": 7}},
+            "right": {"heads": 1, "kv_heads": 1, "dim": 24, "vdim": 72, "conv": 2, "rank": 4},
+            "left_scale": 1.0, "right_scale": 0.5}},
+        {"type": "attention", "mlp": _dense(96), "mixer": {"heads": 4, "kv_heads": 4, "dim": 16, "vdim": 32, "scale": 0.25}},
+        {"type": "attention", "mlp": None, "mixer": {"heads": 8, "kv_heads": 1, "dim": 64, "vdim": 64, "scale": 0.11,
+                                                     "kv_from": 0, "mask": {"size": 33}}},
+    ]}
+
+
+def tiny_config_r():
+    """A width that is no whole 16-byte piece; more first tokens kept than the window is long; a convolution of one tap
+    (no carried inputs); a delta rule wider than a wavefront's columns; five query heads."""
+    return {"architecture": "Tedalix", "vocab": 70, "width": 36, "norm": {"eps": 1e-6, "groups": 2}, "layers": [
+        {"type": "retention", "mlp": _dense(40), "mixer": {"heads": 2, "dim": 12, "vdim": 20, "decay": [0.0, 0.995],
+                                                          "rot": {"base": 100.0, "dims": 12}}},
+        {"type": "attention", "mlp": None, "mixer": {"heads": 5, "kv_heads": 5, "dim": 24, "vdim": 40, "scale": 0.2,
+                                                     "mask": {"size": 8, "keep_first": 30}}},
+        {"type": "parallel", "mlp": _dense(44), "mixer": {
+            "left": {"heads": 5, "kv_heads": 5, "dim": 8, "vdim": 8, "scale": 0.35, "softcap": 5.0, "mask": {"size": 64}},
+            "right": {"heads": 2, "kv_heads": 1, "dim": 48, "vdim": 72, "conv": 1, "rank": 6},
+            "left_scale": 1.3, "right_scale": 1.0}},
+    ]}
