@@ -90,6 +90,32 @@ def test_window_gives_pages_back_early():
     assert t.free_pages(0) == 100 and t.free_pages(1) == 100
 
 
+def test_a_window_that_keeps_the_first_tokens_keeps_their_pages():
+    """Group 0 looks back over 6 keys and every query also sees the first 5: their pages (two of four tokens) stay
+    while the request lives, the pages between them and the window go back, and all return when it ends."""
+    t = PageTables(4, [(12, 6, 5), (12, 6)])
+    assert t.peak_pages(1000, 1, 0) == t.peak_pages(1000, 1, 1) + 2
+    for rid in (1, 2):                      # the second request takes the pages the first gave back
+        t.open(rid)
+        pos = 0
+        for n in (3, 9, 1, 1, 2, 1, 7, 1, 1, 1, 5):
+            t.reserve(rid, pos + n)
+            table = t.table(rid, 0)
+            first_key = max(0, pos - 6 + 1)
+            for key in list(range(min(5, pos + n))) + list(range(first_key, pos + n)):
+                assert table[key // 4] >= 0, f"key {key} lost its page at position {pos}"
+            for i, pg in enumerate(table):
+                if i >= 2 and (i + 1) * 4 <= first_key:
+                    assert pg == -1, f"page {i} is behind the window at position {pos}"
+            pos += n
+            t.commit(rid, pos)
+            assert t.audit() == ""
+        assert t.table(rid, 1)[0] == -1 and t.table(rid, 0)[0] >= 0
+        assert t.live_pages(rid, 0) == t.live_pages(rid, 1) + 2
+        t.close(rid)
+        assert t.free_pages(0) == 12 and t.free_pages(1) == 12
+
+
 def test_all_groups_or_none():
     t = PageTables(4, [(10, 0), (2, 0)])
     t.open(1)
