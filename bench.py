@@ -107,8 +107,12 @@ def fazopel_shape(layers=12, width=2048, vocab=65536):
 
 def fazopel_record(args):
     """Prefill and decode throughput of the Fazopel shape and of the Qwen3 shape beside it, same points."""
-    out = {"arch": "fazopel", "dtype": args.dtype, "layers": args.layers or 12, "points": {}}
-    for name, raw in (("fazopel", fazopel_shape(args.layers or 12)), ("qwen3_beside", qwen3_beside_libodra(args.layers or 12))):
+    return arch_record(args, "fazopel", (("fazopel", fazopel_shape(args.layers or 12)), ("qwen3_beside", qwen3_beside_libodra(args.layers or 12))))
+
+
+def arch_record(args, arch, shapes):
+    out = {"arch": arch, "dtype": args.dtype, "layers": args.layers or 12, "points": {}}
+    for name, raw in shapes:
         pts = {}
         for t in (512, args.prefill_tokens):
             sec = time_prefill(raw, args.dtype, t, reps=3)
@@ -118,6 +122,44 @@ def fazopel_record(args):
             pts[f"decode_b{b}_ctx{ctx}"] = {"ms": round(sec * 1e3, 3), "tok_per_s": round(b / sec, 1)}
         out["points"][name] = pts
     return out
+
+
+# ``--arch tedalix``: a decoder of the Tedalix design at layer sizes of a real model of that kind, in periods of four
+# layers: attention under a window that keeps the first tokens; sink attention beside the gated delta rule; retention
+# (no feed-forward); attention that reads the first layer's keys and values -- beside a Fazopel decoder of the same
+# width, depth, vocabulary, head sizes and dense feed-forwards (three layers of linear attention to one of attention)
+def tedalix_shape(layers=12, width=2048, vocab=65536):
+    heads = 16
+    mask = dict(size=1024, keep_first=4)
+    attention = dict(heads=heads, kv_heads=8, dim=128, vdim=128, scale=128 ** -0.5, mask=mask)
+    parallel = dict(left=dict(heads=heads, kv_heads=4, dim=128, vdim=128, scale=128 ** -0.5, softcap=30.0, mask=dict(size=512)),
+                    right=dict(heads=heads, kv_heads=8, dim=128, vdim=128, conv=4, rank=128), left_scale=0.8, right_scale=0.9)
+    retention = dict(heads=heads, dim=128, vdim=128, rot=dict(base=1000000.0, dims=64),
+                     decay=[1.0 - 2.0 ** -(5.0 + 3.0 * h / heads) for h in range(heads)])
+    dense = dict(kind="dense", ff=8192)
+    out = []
+    for i in range(layers):
+        if i % 4 == 0:
+            out.append(dict(type="attention", mixer=attention, mlp=dense))
+        elif i % 4 == 1:
+            out.append(dict(type="parallel", mixer=parallel, mlp=dense))
+        elif i % 4 == 2:
+            out.append(dict(type="retention", mixer=retention, mlp=None))
+        else:
+            out.append(dict(type="attention", mixer=dict(attention, kv_from=i - 3), mlp=dense))
+    return dict(architecture="Tedalix", vocab=vocab, width=width, norm=dict(eps=1e-6, groups=4), layers=out)
+
+
+def fazopel_beside_tedalix(layers=12):
+    raw = fazopel_shape(layers)
+    for lc in raw["layers"]:
+        lc["mlp"] = dict(kind="dense", ff=8192)
+    return raw
+
+
+def tedalix_record(args):
+    """Prefill and decode throughput of the Tedalix shape and of a dense Fazopel shape beside it, same points."""
+    return arch_record(args, "tedalix", (("tedalix", tedalix_shape(args.layers or 12)), ("fazopel_beside", fazopel_beside_tedalix(args.layers or 12))))
 
 
 def build_engine(raw, dtype, cache_tokens, seed=0, page_size=16, **cfg_overrides):
@@ -355,8 +397,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has (named in config)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--shape", default="4b", choices=sorted(SHAPES), help="layer sizes: Qwen3-4B (the default run), 0.6B, 8B or 32B")
-    ap.add_argument("--arch", default="qwen3", choices=["qwen3", "libodra", "fazopel"],
-                    help="libodra, fazopel: prefill and decode of that design at a real model's layer sizes beside a Qwen3 "
+    ap.add_argument("--arch", default="qwen3", choices=["qwen3", "libodra", "fazopel", "tedalix"],
+                    help="libodra, fazopel, tedalix: prefill and decode of that design at a real model's layer sizes beside the closest other "
                          "decoder of equal size, as one record (the default run and its record are Qwen3's)")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the points at other batches and lengths")
@@ -385,6 +427,9 @@ def main() -> int:
         return 0
     if args.arch == "fazopel":
         print(json.dumps(fazopel_record(args)), flush=True)
+        return 0
+    if args.arch == "tedalix":
+        print(json.dumps(tedalix_record(args)), flush=True)
         return 0
     raw = dict(SHAPES[args.shape])
     name = f"Qwen3-{args.shape.upper()} shape"
