@@ -156,6 +156,110 @@ __global__ __launch_bounds__(kWave) void gated_delta_kernel(const float* __restr
   }
 }
 
+// The recurrence for portions of prompts: the same sums with a column of S spread over R neighbouring lanes, each
+// keeping D / R rows in registers (four consecutive rows of every R-th group of four, so that the R lanes of a column read
+// one contiguous stretch of LDS), and the two dot products summed across the R lanes inside the wavefront's rows of 16
+// lanes.  A sequence of one head is then 256 / R columns a workgroup instead of 64 a wavefront: sixteen times the
+// wavefronts, and a dependent chain of D / R instead of D multiply-adds a token.  The order of every sum still follows
+// the token's place alone.
+template <int R>
+__device__ __forceinline__ float sum_over_lanes(float v) {
+  static_assert(R == 8 || R == 16, "a column's lanes lie inside a row of 16");
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));    // lane ^ 1
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));    // lane ^ 2
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));   // 7 - lane within eight
+  if (R == 16) v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));   // 15 - lane
+  return v;
+}
+
+template <int D, int R>
+__global__ __launch_bounds__(256) void gated_delta_rows_kernel(const float* __restrict__ x, const float* __restrict__ decay,
+                                                               const float* __restrict__ beta, float* __restrict__ state,
+                                                               const int* __restrict__ state_slots, const int* __restrict__ cu_q,
+                                                               float* __restrict__ out, int heads, int kvh, int d, int e) {
+  constexpr int NT = 16;            // tokens staged at a time
+  constexpr int NV = D / R / 4;     // groups of four rows a lane keeps
+  constexpr int COLS = 256 / R;
+  static_assert(D % (4 * R) == 0, "a lane keeps whole groups of four rows");
+  __shared__ float4 ks[NT][D / 4], qs[NT][D / 4], gs[NT][D / 4];
+  __shared__ float bs[NT];
+  const int seq = blockIdx.x, h = blockIdx.y;
+  const int rho = threadIdx.x % R;
+  const int col = blockIdx.z * COLS + threadIdx.x / R;
+  const bool live = col < e;
+  const int begin = cu_q[seq], end = cu_q[seq + 1];
+  if (end <= begin) return;
+  const int kh = h / (heads / kvh);
+  const int qk = kvh * d, C = 2 * qk + heads * e;
+  float* S = state + (((size_t)state_slots[seq] * heads + h) * d) * e;
+  float s[NV][4];
+#pragma unroll
+  for (int i = 0; i < NV; ++i)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int j = 4 * (i * R + rho) + c;
+      s[i][c] = (live && j < d) ? S[(size_t)j * e + col] : 0.f;
+    }
+  for (int t0 = begin; t0 < end; t0 += NT) {
+    const int n = end - t0 < NT ? end - t0 : NT;
+    __syncthreads();
+    for (int i = threadIdx.x; i < n * D; i += 256) {
+      const int tk = i / D, j = i % D;
+      const size_t t = t0 + tk;
+      const bool in = j < d;
+      reinterpret_cast<float*>(qs[tk])[j] = in ? x[t * C + kh * d + j] : 0.f;
+      reinterpret_cast<float*>(ks[tk])[j] = in ? x[t * C + qk + kh * d + j] : 0.f;
+      reinterpret_cast<float*>(gs[tk])[j] = in ? decay[(t * heads + h) * d + j] : 1.f;
+    }
+    if (threadIdx.x < n) bs[threadIdx.x] = beta[(size_t)(t0 + threadIdx.x) * heads + h];
+    __syncthreads();
+    float v[NT];
+#pragma unroll
+    for (int tk = 0; tk < NT; ++tk) v[tk] = (live && tk < n) ? x[(size_t)(t0 + tk) * C + 2 * qk + h * e + col] : 0.f;
+#pragma unroll
+    for (int tk = 0; tk < NT; ++tk) {
+      if (tk < n) {
+        float4 kk[NV];
+        float part[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+          const float4 gg = gs[tk][i * R + rho];
+          kk[i] = ks[tk][i * R + rho];
+          s[i][0] *= gg.x; s[i][1] *= gg.y; s[i][2] *= gg.z; s[i][3] *= gg.w;
+          part[0] = fmaf(s[i][0], kk[i].x, part[0]);
+          part[1] = fmaf(s[i][1], kk[i].y, part[1]);
+          part[2] = fmaf(s[i][2], kk[i].z, part[2]);
+          part[3] = fmaf(s[i][3], kk[i].w, part[3]);
+        }
+        const float kv = sum_over_lanes<R>((part[0] + part[1]) + (part[2] + part[3]));
+        const float u = bs[tk] * (v[tk] - kv);
+        float po[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+          const float4 qq = qs[tk][i * R + rho];
+          s[i][0] = fmaf(kk[i].x, u, s[i][0]); s[i][1] = fmaf(kk[i].y, u, s[i][1]);
+          s[i][2] = fmaf(kk[i].z, u, s[i][2]); s[i][3] = fmaf(kk[i].w, u, s[i][3]);
+          po[0] = fmaf(s[i][0], qq.x, po[0]);
+          po[1] = fmaf(s[i][1], qq.y, po[1]);
+          po[2] = fmaf(s[i][2], qq.z, po[2]);
+          po[3] = fmaf(s[i][3], qq.w, po[3]);
+        }
+        const float o = sum_over_lanes<R>((po[0] + po[1]) + (po[2] + po[3]));
+        if (live && rho == 0) out[((size_t)(t0 + tk) * heads + h) * e + col] = o;
+      }
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int j = 4 * (i * R + rho) + c;
+        if (j < d) S[(size_t)j * e + col] = s[i][c];
+      }
+  }
+}
+
 // p [T, stride] -> out [T, 2 * heads * d + heads * e] 32-bit: queries (from q_off) and keys (from k_off) with the
 // first `rot` dimensions of every head turned, dimension i with i + rot / 2, by positions[t] * inv_freq[i]; the keys
 // then times k_scale; values (from v_off) as they are.  A thread an element (a pair's two ends are two threads).
@@ -228,13 +332,24 @@ extern "C" int pa_delta_prepare(void* stream, int dtype, const void* p, long str
 }
 
 extern "C" int pa_gated_delta(void* stream, const float* x, const float* decay, const float* beta, float* state,
-                              const int* state_slots, const int* cu_q, float* out, int nseq, int heads, int kvh, int d, int e) {
+                              const int* state_slots, const int* cu_q, float* out, int nseq, int heads, int kvh, int d, int e,
+                              int portions) {
   if (nseq == 0) return 0;
   PA_REQUIRE(nseq > 0 && heads > 0 && kvh > 0 && heads % kvh == 0 && d > 0 && e > 0,
              "gated_delta: bad sizes sequences=%d heads=%d key heads=%d d=%d e=%d", nseq, heads, kvh, d, e);
   PA_REQUIRE(d <= 256, "gated_delta: a key width of %d is more than the 256 the kernel takes", d);
-  dim3 grid(nseq, heads, (e + kWave - 1) / kWave);
   hipStream_t st = (hipStream_t)stream;
+  if (portions) {   // some sequence brings more than a token: a column over several lanes
+#define PA_DELTA_ROWS(D, R) hipLaunchKernelGGL((gated_delta_rows_kernel<D, R>), dim3(nseq, heads, (e + 256 / R - 1) / (256 / R)), dim3(256), \
+                                               0, st, x, decay, beta, state, state_slots, cu_q, out, heads, kvh, d, e)
+    if (d <= 32) PA_DELTA_ROWS(32, 8);
+    else if (d <= 64) PA_DELTA_ROWS(64, 16);
+    else if (d <= 128) PA_DELTA_ROWS(128, 16);
+    else PA_DELTA_ROWS(256, 16);
+#undef PA_DELTA_ROWS
+    return check_launch("gated_delta");
+  }
+  dim3 grid(nseq, heads, (e + kWave - 1) / kWave);
 #define PA_DELTA(D) hipLaunchKernelGGL(gated_delta_kernel<D>, grid, dim3(kWave), 0, st, x, decay, beta, state, state_slots, cu_q, \
                                        out, heads, kvh, d, e)
   if (d <= 32) PA_DELTA(32);

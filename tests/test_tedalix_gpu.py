@@ -230,6 +230,59 @@ def test_queries_and_keys_normed_over_the_whole_projection(gpu, dtype, nh, nkv, 
     close(only_q.reshape(T, nq), wq, dtype, "queries of a layer that reads another's keys")
 
 
+# ---- the gated delta rule's recurrence alone ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("singles", [False, True])
+@pytest.mark.parametrize("heads,kvh,d,e", [(4, 2, 16, 24), (2, 1, 48, 72), (4, 4, 32, 32), (3, 1, 20, 8), (1, 1, 8, 136), (2, 2, 256, 64),
+                                           (8, 4, 128, 128), (2, 1, 100, 40)])
+def test_the_delta_rule_alone(gpu, heads, kvh, d, e, singles):
+    """Unequal sequences in one launch, each from a state of its own in a slot of its own: outputs and the states left
+    behind, for steps with portions (a column of the state over several lanes) and steps of single tokens alone (a lane
+    a column).  A key written once with beta 1 and no decay is read back by the same query, overwritten by the next
+    writes under the same key."""
+    from prelude_amd.ops import kernels as K
+    lengths = [1, 1, 1] if singles else [1, 47, 16, 17, 2, 33]
+    slots = [4, 0, 6] if singles else [7, 2, 5, 0, 4, 1]
+    T = sum(lengths)
+    g = torch.Generator().manual_seed(81)
+    q = torch.randn((T, kvh, d), generator=g)
+    k = torch.randn((T, kvh, d), generator=g)
+    q = q / q.norm(dim=-1, keepdim=True) * d ** -0.5
+    k = k / k.norm(dim=-1, keepdim=True)
+    v = torch.randn((T, heads, e), generator=g)
+    decay = torch.rand((T, heads, d), generator=g) * 0.3 + 0.7
+    beta = torch.rand((T, heads), generator=g)
+    if not singles:                       # the second sequence: a write that is read back and overwritten
+        k[3] = k[2]; q[3] = k[2]; k[4] = k[2]; q[4] = k[2]
+        beta[2:5] = 1.0
+        decay[3:5] = 1.0
+    state0 = torch.randn((8, heads, d, e), generator=g)
+    state = state0.to(gpu)
+    x = torch.cat([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], dim=1).contiguous()
+    cu = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    step = types.SimpleNamespace(num_seqs=len(lengths), cu_q=torch.tensor(cu, device=gpu),
+                                 state_slots=torch.tensor(slots, dtype=torch.int32, device=gpu))
+    out = K.gated_delta(x.to(gpu), decay.to(gpu), beta.to(gpu), state, step, heads, kvh, d, e)
+    want = torch.zeros((T, heads, e), dtype=torch.float64)
+    row = 0
+    for n, slot in zip(lengths, slots):
+        for h in range(heads):
+            kh = h // (heads // kvh)
+            S = state0[slot, h].double()
+            for t in range(row, row + n):
+                S = decay[t, h].double()[:, None] * S
+                u = beta[t, h].double() * (v[t, h].double() - S.T @ k[t, kh].double())
+                S = S + torch.outer(k[t, kh].double(), u)
+                want[t, h] = S.T @ q[t, kh].double()
+            close(state[slot, h], S, "float32", f"the state of slot {slot}, head {h}", scale=float(state0.abs().max()))
+        row += n
+    close(out, want, "float32", "outputs", scale=float(want.abs().max()))
+    if not singles:
+        close(out[3], v[3].double(), "float32", "a second write under the same key is read back in place of the first")
+        close(out[4], v[4].double(), "float32", "and a third")
+    untouched = [i for i in range(8) if i not in slots]
+    assert torch.equal(state[untouched].cpu(), state0[untouched]), "other requests' states are left alone"
+
+
 # ---- one-layer models: every mixer alone through the engine ------------------------------------------------------------------
 def _dense(ff):
     return {"kind": "dense", "ff": ff}
