@@ -108,7 +108,8 @@ _KERNEL_API = {
     "pa_group_norm_step": (I, [P, I, P, P, P, P, P, P, I, I, I, F]),
     "pa_poly_norm": (I, [P, I, P, P, P, P, I, I, F]),
     "pa_head_norm_gate": (I, [P, I, P, P, c_long, P, P, c_long, I, I, I, F, I, F]),
-    "pa_attn_masked": (I, [P, I, P, P, P, P, I, P, P, P, c_long, I, I, I, I, I, I, I, I, F, F, P, P, P, c_long, F]),
+    "pa_attn_masked": (I, [P, I, P, P, P, P, I, P, P, P, c_long, I, I, I, I, I, I, I, I, F, F, P, P, P, c_long, F, P, P, I, I]),
+    "pa_attn_masked_mfma_supports": (I, [I, I, I]),
     "pa_qkv_prepare": (I, [P, I, P, c_long, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, F]),
     "pa_delta_prepare": (I, [P, I, P, c_long, I, I, P, I, P, P, P, P, P, c_long, I, P, P, P, P, P, I, I, I, I, I, I]),
     "pa_gated_delta": (I, [P, P, P, P, P, P, P, P, I, I, I, I, I, I]),

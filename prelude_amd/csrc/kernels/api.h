@@ -300,7 +300,9 @@ int pa_head_norm_gate(void* stream, int dtype, const float* o, const void* gate,
 int pa_attn_masked(void* stream, int dtype, const void* q, const void* k_cache, const void* v_cache, const int* block_table,
                    int table_stride, const int* seq_of_token, const int* positions, void* out, long out_stride, int tokens,
                    int nh, int nkv, int hd, int vd, int page_size, int window, int keep_first, float scale, float softcap,
-                   const float* slopes, const float* sink, const void* gate, long gate_stride, float out_scale);
+                   const float* slopes, const float* sink, const void* gate, long gate_stride, float out_scale, const int* cu_q,
+                   const int* context_lens, int nseq, int max_q_len);
+int pa_attn_masked_mfma_supports(int hd, int vd, int page_size);
 int pa_qkv_prepare(void* stream, int dtype, const void* p, long stride, int q_off, int k_off, int v_off, const float* qw,
                    const float* kw, const int* slots, void* q_out, void* k_cache, void* v_cache, int tokens, int nh, int nkv,
                    int hd, int vd, int page_size, float eps);

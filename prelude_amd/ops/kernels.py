@@ -1686,7 +1686,11 @@ def attention_masked(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     to cap * tanh(score / cap) for ``softcap`` > 0, less ``slopes``[h] * (i - j); ``sink`` [heads] joins the softmax's
     denominator; ``gate`` [T, heads] (rows may lie inside a wider tensor): a head's output times sigmoid(gate), and
     ``out_scale``, before rounding.  q [T, nh, hd]; K cache [pages, nkv, page, hd]; V cache [pages, nkv, vd, page].
-    Returns (or fills ``out``, whose rows may lie inside a wider tensor) [T, nh * vd]."""
+    Returns (or fills ``out``, whose rows may lie inside a wider tensor) [T, nh * vd].
+
+    bfloat16 with keys and values of one width the matrix cores take (32, 64, 96, 128) and pages of a power of two runs
+    on the matrix cores: portions as tiles of 64 tokens, a single token's keys dealt out to a workgroup's wavefronts.
+    Everything else (32-bit, other sizes) runs on the vector units, a wavefront a (token, head)."""
     _dev(q, k_cache, v_cache, slopes, sink)
     if q.dim() != 3 or not q.is_contiguous() or k_cache.dim() != 4 or v_cache.dim() != 4:
         raise NativeError(f"attention_masked: q {tuple(q.shape)} / caches")
@@ -1711,7 +1715,9 @@ def attention_masked(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                                        group.block_table.shape[1], _ptr(step.seq_of_token), _ptr(step.positions), out.data_ptr(),
                                        out.stride(0), t, nh, nkv, hd, vd, page, int(window), int(keep_first), float(scale),
                                        float(softcap), _ptr(slopes), _ptr(sink), gate.data_ptr() if gate is not None else None,
-                                       gate.stride(0) if gate is not None else 0, float(out_scale)))
+                                       gate.stride(0) if gate is not None else 0, float(out_scale), _ptr(getattr(step, "cu_q", None)),
+                                       _ptr(getattr(step, "context_lens", None)), int(getattr(step, "num_seqs", 0)),
+                                       int(getattr(step, "max_q_len", 0) or getattr(step, "max_prefill_q", 0) or 1)))
     return out
 
 
