@@ -23,7 +23,7 @@
 //
 // In bfloat16, with keys and values of 32, 64, 96 or 128 and pages of a power of two, the same attention runs on the
 // matrix cores (`attn_masked_mfma_kernel` below), with the inner step of the plain matrix-core kernels: a wavefront
-// owns 16 tokens of up to four heads that share a KV head and walks, 32 keys a step, first the steps that hold kept
+// owns 16 tokens of two heads that share a KV head (one when the group is odd) and walks, 32 keys a step, first the steps that hold kept
 // first tokens and then the window's; a sequence that brings one token has its steps dealt out to the workgroup's
 // four wavefronts, whose sums are merged through LDS.
 #include "common.h"
@@ -187,9 +187,12 @@ __device__ __forceinline__ void attend32_masked(const KeyWalk& w, int kept, int 
 #pragma unroll
       for (int i = 0; i < 4; ++i) s[4 * t + i] = acc[i];
     }
-    if (sm.cap != 0.f) {
+    if (sm.cap != 0.f) {   // tanh(x) = 1 - 2 / (1 + e^(2x)), with the hardware's exponential and reciprocal
 #pragma unroll
-      for (int i = 0; i < 8; ++i) s[i] = sm.cap * tanhf(s[i] * sm.cap_in);
+      for (int i = 0; i < 8; ++i) {
+        const float e2 = __builtin_amdgcn_exp2f(s[i] * sm.cap_in * (2.0f * kLog2e));
+        s[i] = sm.cap - 2.0f * sm.cap * __builtin_amdgcn_rcpf(1.0f + e2);
+      }
     }
     if (bias[j] != 0.f) {
       const float d0 = (float)(my_pos - (key0 + 8 * g));
@@ -442,18 +445,18 @@ extern "C" int pa_attn_masked(void* stream, int dtype, const void* q, const void
   hipStream_t st = (hipStream_t)stream;
   if (dtype == kBF16 && pa_attn_masked_mfma_supports(hd, vd, page_size) && cu_q && context_lens && nseq > 0 && max_q_len > 0) {
     const int group = nh / nkv;
-    const int gt = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
+    // two heads a wavefront where the group is even: four leave a head of 128 no registers and measured slower
+    const int gt = group % 2 == 0 ? 2 : 1;
     MaskedArgs a{(const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache, block_table, table_stride, cu_q, context_lens,
                  (bf16*)out, (size_t)out_stride, nh, nkv, __builtin_ctz(page_size), window, window > 0 ? keep_first : 0,
                  score_map(scale, softcap, sink), softcap > 0.f ? 1.0f : 1.0f / scale, slopes, (const bf16*)gate,
                  (size_t)gate_stride, out_scale};
     dim3 mgrid((max_q_len + 63) / 64, nkv * (group / gt), nseq);
 #define PA_MASKED(D, GT) hipLaunchKernelGGL((attn_masked_mfma_kernel<D, D, GT>), mgrid, dim3(256), 0, st, a)
-#define PA_MASKED_GT(D)          \
-  do {                           \
-    if (gt == 4) PA_MASKED(D, 4); \
-    else if (gt == 2) PA_MASKED(D, 2); \
-    else PA_MASKED(D, 1);        \
+#define PA_MASKED_GT(D)              \
+  do {                               \
+    if (gt == 2) PA_MASKED(D, 2);    \
+    else PA_MASKED(D, 1);            \
   } while (0)
     if (hd == 32) PA_MASKED_GT(32);
     else if (hd == 64) PA_MASKED_GT(64);

@@ -102,6 +102,61 @@ __global__ __launch_bounds__(kRowThreads) void poly_norm_kernel(const T* __restr
   }
 }
 
+// The same for bfloat16 rows of a multiple of 8 up to 8 * 256 * VPT elements: a thread keeps its pieces of 8 elements
+// (with the bias added, in 32-bit) in registers, so the row is read once, in 16-byte loads.
+template <int VPT>
+__global__ __launch_bounds__(256) void poly_norm_vec_kernel(const bf16* __restrict__ x, const float* __restrict__ bias,
+                                                            const float* __restrict__ coeff, bf16* __restrict__ out, int width,
+                                                            float eps) {
+  __shared__ float scratch[16];
+  const size_t r = blockIdx.x;
+  const bf16* xr = x + r * width;
+  const int pieces = width / 8;
+  float z[VPT][8];
+  float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+#pragma unroll
+  for (int v = 0; v < VPT; ++v) {
+    const int piece = v * 256 + threadIdx.x;
+    if (piece < pieces) {
+      const bf16x8 raw = *reinterpret_cast<const bf16x8*>(xr + 8 * piece);
+      float4 b0{0.f, 0.f, 0.f, 0.f}, b1{0.f, 0.f, 0.f, 0.f};
+      if (bias) {
+        b0 = *reinterpret_cast<const float4*>(bias + 8 * piece);
+        b1 = *reinterpret_cast<const float4*>(bias + 8 * piece + 4);
+      }
+      const float bb[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        z[v][i] = (float)raw[i] + bb[i];
+        const float z2 = z[v][i] * z[v][i];
+        s2 += z2;
+        s4 += z2 * z2;
+        s6 += z2 * z2 * z2;
+      }
+    }
+  }
+  s2 = block_sum(s2, scratch);
+  s4 = block_sum(s4, scratch);
+  s6 = block_sum(s6, scratch);
+  const float n = (float)width;
+  const float a = coeff[0] / sqrtf(s2 / n + eps), b = coeff[1] / sqrtf(s4 / n + eps), c = coeff[2] / sqrtf(s6 / n + eps);
+  const float e = coeff[3];
+  bf16* dst = out + r * width;
+#pragma unroll
+  for (int v = 0; v < VPT; ++v) {
+    const int piece = v * 256 + threadIdx.x;
+    if (piece < pieces) {
+      bf16x8 o;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float zz = z[v][i];
+        o[i] = (bf16)(a * zz + b * (zz * zz) + c * (zz * zz * zz) + e);
+      }
+      *reinterpret_cast<bf16x8*>(dst + 8 * piece) = o;
+    }
+  }
+}
+
 // A wavefront a (row, head): out[r, h, :] = o[r, h, :] / sqrt(mean(o[r, h, :]^2) + eps) * w * act(gate[r, h, :]) * scale.
 // w (or null: no weight) has `vdim` elements shared by the heads; gate act: 0 sigmoid(g), 1 g * sigmoid(g).
 template <typename T>
@@ -164,7 +219,16 @@ extern "C" int pa_poly_norm(void* stream, int dtype, const void* x, const float*
   if (dtype == kF32)
     hipLaunchKernelGGL(poly_norm_kernel<float>, dim3(nrows), dim3(kRowThreads), 0, st, (const float*)x, bias, coeff,
                        (float*)out, width, eps);
-  else if (dtype == kBF16)
+  else if (dtype == kBF16 && width % 8 == 0 && width <= 8 * 256 * 8 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+           (reinterpret_cast<uintptr_t>(out) & 15) == 0 && (reinterpret_cast<uintptr_t>(bias) & 15) == 0) {
+    const int vpt = (width / 8 + 255) / 256;
+#define PA_POLY(V) hipLaunchKernelGGL(poly_norm_vec_kernel<V>, dim3(nrows), dim3(256), 0, st, (const bf16*)x, bias, coeff, (bf16*)out, width, eps)
+    if (vpt <= 1) PA_POLY(1);
+    else if (vpt <= 2) PA_POLY(2);
+    else if (vpt <= 4) PA_POLY(4);
+    else PA_POLY(8);
+#undef PA_POLY
+  } else if (dtype == kBF16)
     hipLaunchKernelGGL(poly_norm_kernel<bf16>, dim3(nrows), dim3(kRowThreads), 0, st, (const bf16*)x, bias, coeff, (bf16*)out,
                        width, eps);
   else
