@@ -172,17 +172,23 @@ __device__ __forceinline__ float sum_over_lanes(float v) {
   return v;
 }
 
-template <int D, int R>
+// Tokens go through LDS NT at a time, in two buffers: the next NT are asked for (16-byte pieces where the key width
+// and the row allow, VEC) before the current ones are worked through and put into the other buffer afterwards, one
+// barrier a block of tokens.  Places past a sequence's end or past the key width hold k = q = 0, g = 1, beta = 0,
+// which leave the state as it is: the walk over a block's tokens has no branch, so the reads of the next token's
+// rows can run ahead of the sums of this one.
+template <int D, int R, bool VEC>
 __global__ __launch_bounds__(256) void gated_delta_rows_kernel(const float* __restrict__ x, const float* __restrict__ decay,
                                                                const float* __restrict__ beta, float* __restrict__ state,
                                                                const int* __restrict__ state_slots, const int* __restrict__ cu_q,
                                                                float* __restrict__ out, int heads, int kvh, int d, int e) {
-  constexpr int NT = 16;            // tokens staged at a time
-  constexpr int NV = D / R / 4;     // groups of four rows a lane keeps
+  constexpr int NT = D <= 128 ? 16 : 8;   // tokens staged at a time
+  constexpr int NV = D / R / 4;           // groups of four rows a lane keeps
   constexpr int COLS = 256 / R;
+  constexpr int PER = (NT * (D / 4) + 255) / 256;   // 16-byte pieces of each staged array a thread moves
   static_assert(D % (4 * R) == 0, "a lane keeps whole groups of four rows");
-  __shared__ float4 ks[NT][D / 4], qs[NT][D / 4], gs[NT][D / 4];
-  __shared__ float bs[NT];
+  __shared__ float4 ks[2][NT][D / 4], qs[2][NT][D / 4], gs[2][NT][D / 4];
+  __shared__ float bs[2][NT];
   const int seq = blockIdx.x, h = blockIdx.y;
   const int rho = threadIdx.x % R;
   const int col = blockIdx.z * COLS + threadIdx.x / R;
@@ -200,54 +206,102 @@ __global__ __launch_bounds__(256) void gated_delta_rows_kernel(const float* __re
       const int j = 4 * (i * R + rho) + c;
       s[i][c] = (live && j < d) ? S[(size_t)j * e + col] : 0.f;
     }
-  for (int t0 = begin; t0 < end; t0 += NT) {
-    const int n = end - t0 < NT ? end - t0 : NT;
-    __syncthreads();
-    for (int i = threadIdx.x; i < n * D; i += 256) {
-      const int tk = i / D, j = i % D;
-      const size_t t = t0 + tk;
-      const bool in = j < d;
-      reinterpret_cast<float*>(qs[tk])[j] = in ? x[t * C + kh * d + j] : 0.f;
-      reinterpret_cast<float*>(ks[tk])[j] = in ? x[t * C + qk + kh * d + j] : 0.f;
-      reinterpret_cast<float*>(gs[tk])[j] = in ? decay[(t * heads + h) * d + j] : 1.f;
-    }
-    if (threadIdx.x < n) bs[threadIdx.x] = beta[(size_t)(t0 + threadIdx.x) * heads + h];
-    __syncthreads();
-    float v[NT];
+  float4 rq[PER], rk[PER], rg[PER];
+  float rb = 0.f;
+  float v[NT], v_next[NT];
+  auto fetch = [&](int t0) {
 #pragma unroll
-    for (int tk = 0; tk < NT; ++tk) v[tk] = (live && tk < n) ? x[(size_t)(t0 + tk) * C + 2 * qk + h * e + col] : 0.f;
+    for (int p = 0; p < PER; ++p) {
+      const int piece = p * 256 + threadIdx.x;
+      const int tk = piece / (D / 4), j = 4 * (piece % (D / 4));
+      const size_t t = (size_t)t0 + tk;
+      rq[p] = rk[p] = float4{0.f, 0.f, 0.f, 0.f};
+      rg[p] = float4{1.f, 1.f, 1.f, 1.f};
+      if (tk < NT && t < (size_t)end) {
+        const float* qp = x + t * C + kh * d + j;
+        const float* kp = qp + qk;
+        const float* gp = decay + (t * heads + h) * d + j;
+        if (VEC) {
+          if (j < d) {
+            rq[p] = *reinterpret_cast<const float4*>(qp);
+            rk[p] = *reinterpret_cast<const float4*>(kp);
+            rg[p] = *reinterpret_cast<const float4*>(gp);
+          }
+        } else {
+          float* fq = reinterpret_cast<float*>(&rq[p]);
+          float* fk = reinterpret_cast<float*>(&rk[p]);
+          float* fg = reinterpret_cast<float*>(&rg[p]);
 #pragma unroll
-    for (int tk = 0; tk < NT; ++tk) {
-      if (tk < n) {
-        float4 kk[NV];
-        float part[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-          const float4 gg = gs[tk][i * R + rho];
-          kk[i] = ks[tk][i * R + rho];
-          s[i][0] *= gg.x; s[i][1] *= gg.y; s[i][2] *= gg.z; s[i][3] *= gg.w;
-          part[0] = fmaf(s[i][0], kk[i].x, part[0]);
-          part[1] = fmaf(s[i][1], kk[i].y, part[1]);
-          part[2] = fmaf(s[i][2], kk[i].z, part[2]);
-          part[3] = fmaf(s[i][3], kk[i].w, part[3]);
+          for (int c = 0; c < 4; ++c)
+            if (j + c < d) {
+              fq[c] = qp[c];
+              fk[c] = kp[c];
+              fg[c] = gp[c];
+            }
         }
-        const float kv = sum_over_lanes<R>((part[0] + part[1]) + (part[2] + part[3]));
-        const float u = bs[tk] * (v[tk] - kv);
-        float po[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-          const float4 qq = qs[tk][i * R + rho];
-          s[i][0] = fmaf(kk[i].x, u, s[i][0]); s[i][1] = fmaf(kk[i].y, u, s[i][1]);
-          s[i][2] = fmaf(kk[i].z, u, s[i][2]); s[i][3] = fmaf(kk[i].w, u, s[i][3]);
-          po[0] = fmaf(s[i][0], qq.x, po[0]);
-          po[1] = fmaf(s[i][1], qq.y, po[1]);
-          po[2] = fmaf(s[i][2], qq.z, po[2]);
-          po[3] = fmaf(s[i][3], qq.w, po[3]);
-        }
-        const float o = sum_over_lanes<R>((po[0] + po[1]) + (po[2] + po[3]));
-        if (live && rho == 0) out[((size_t)(t0 + tk) * heads + h) * e + col] = o;
       }
     }
+    rb = (threadIdx.x < NT && t0 + (int)threadIdx.x < end) ? beta[(size_t)(t0 + threadIdx.x) * heads + h] : 0.f;
+#pragma unroll
+    for (int tk = 0; tk < NT; ++tk) v_next[tk] = (live && t0 + tk < end) ? x[(size_t)(t0 + tk) * C + 2 * qk + h * e + col] : 0.f;
+  };
+  auto put = [&](int buf) {
+#pragma unroll
+    for (int p = 0; p < PER; ++p) {
+      const int piece = p * 256 + threadIdx.x;
+      if (piece < NT * (D / 4)) {
+        (&qs[buf][0][0])[piece] = rq[p];
+        (&ks[buf][0][0])[piece] = rk[p];
+        (&gs[buf][0][0])[piece] = rg[p];
+      }
+    }
+    if (threadIdx.x < NT) bs[buf][threadIdx.x] = rb;
+  };
+  fetch(begin);
+  put(0);
+#pragma unroll
+  for (int tk = 0; tk < NT; ++tk) v[tk] = v_next[tk];
+  __syncthreads();
+  int buf = 0;
+  for (int t0 = begin; t0 < end; t0 += NT, buf ^= 1) {
+    const bool more = t0 + NT < end;
+    if (more) fetch(t0 + NT);
+#pragma unroll
+    for (int tk = 0; tk < NT; ++tk) {
+      float4 kk[NV];
+      float part[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const float4 gg = gs[buf][tk][i * R + rho];
+        kk[i] = ks[buf][tk][i * R + rho];
+        s[i][0] *= gg.x; s[i][1] *= gg.y; s[i][2] *= gg.z; s[i][3] *= gg.w;
+        part[0] = fmaf(s[i][0], kk[i].x, part[0]);
+        part[1] = fmaf(s[i][1], kk[i].y, part[1]);
+        part[2] = fmaf(s[i][2], kk[i].z, part[2]);
+        part[3] = fmaf(s[i][3], kk[i].w, part[3]);
+      }
+      const float kv = sum_over_lanes<R>((part[0] + part[1]) + (part[2] + part[3]));
+      const float u = bs[buf][tk] * (v[tk] - kv);
+      float po[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const float4 qq = qs[buf][tk][i * R + rho];
+        s[i][0] = fmaf(kk[i].x, u, s[i][0]); s[i][1] = fmaf(kk[i].y, u, s[i][1]);
+        s[i][2] = fmaf(kk[i].z, u, s[i][2]); s[i][3] = fmaf(kk[i].w, u, s[i][3]);
+        po[0] = fmaf(s[i][0], qq.x, po[0]);
+        po[1] = fmaf(s[i][1], qq.y, po[1]);
+        po[2] = fmaf(s[i][2], qq.z, po[2]);
+        po[3] = fmaf(s[i][3], qq.w, po[3]);
+      }
+      const float o = sum_over_lanes<R>((po[0] + po[1]) + (po[2] + po[3]));
+      if (live && rho == 0 && t0 + tk < end) out[((size_t)(t0 + tk) * heads + h) * e + col] = o;
+    }
+    if (more) {
+      put(buf ^ 1);
+#pragma unroll
+      for (int tk = 0; tk < NT; ++tk) v[tk] = v_next[tk];
+    }
+    __syncthreads();
   }
   if (live) {
 #pragma unroll
@@ -340,8 +394,19 @@ extern "C" int pa_gated_delta(void* stream, const float* x, const float* decay, 
   PA_REQUIRE(d <= 256, "gated_delta: a key width of %d is more than the 256 the kernel takes", d);
   hipStream_t st = (hipStream_t)stream;
   if (portions) {   // some sequence brings more than a token: a column over several lanes
-#define PA_DELTA_ROWS(D, R) hipLaunchKernelGGL((gated_delta_rows_kernel<D, R>), dim3(nseq, heads, (e + 256 / R - 1) / (256 / R)), dim3(256), \
-                                               0, st, x, decay, beta, state, state_slots, cu_q, out, heads, kvh, d, e)
+    // 16-byte loads of queries, keys and decays where every row of them starts at a multiple of four floats
+    const bool vec = d % 4 == 0 && (2 * kvh * d + heads * e) % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+                     (reinterpret_cast<uintptr_t>(decay) & 15) == 0;
+#define PA_DELTA_ROWS(D, R)                                                                                                       \
+  do {                                                                                                                            \
+    dim3 rgrid(nseq, heads, (e + 256 / R - 1) / (256 / R));                                                                       \
+    if (vec)                                                                                                                      \
+      hipLaunchKernelGGL((gated_delta_rows_kernel<D, R, true>), rgrid, dim3(256), 0, st, x, decay, beta, state, state_slots, cu_q, \
+                         out, heads, kvh, d, e);                                                                                  \
+    else                                                                                                                          \
+      hipLaunchKernelGGL((gated_delta_rows_kernel<D, R, false>), rgrid, dim3(256), 0, st, x, decay, beta, state, state_slots,      \
+                         cu_q, out, heads, kvh, d, e);                                                                            \
+  } while (0)
     if (d <= 32) PA_DELTA_ROWS(32, 8);
     else if (d <= 64) PA_DELTA_ROWS(64, 16);
     else if (d <= 128) PA_DELTA_ROWS(128, 16);
