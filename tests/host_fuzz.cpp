@@ -10,7 +10,7 @@
 #include <string>
 #include <vector>
 extern "C" {
-void* pa_cache_create(int, int, const int*, const int*, int);
+void* pa_cache_create(int, int, const int*, const int*, const int*, int);
 void pa_cache_destroy(void*);
 int pa_cache_open(void*, long long, int);
 int pa_cache_reserve(void*, long long, int);
@@ -46,10 +46,14 @@ int main(int argc, char** argv) {
     auto R = [&](int lo, int hi) { return lo + (int)(rng() % (unsigned)(hi - lo + 1)); };
     const int page = 1 << R(0, 5);
     const int groups = R(1, 3);
-    int pages[3], windows[3];
-    for (int g = 0; g < groups; ++g) { pages[g] = R(0, 3) ? R(4, 40) : R(8, 200); windows[g] = R(0, 2) == 0 ? R(1, 300) : 0; }
+    int pages[3], windows[3], kept[3];
+    for (int g = 0; g < groups; ++g) {
+      pages[g] = R(0, 3) ? R(4, 40) : R(8, 200);
+      windows[g] = R(0, 2) == 0 ? R(1, 300) : 0;
+      kept[g] = (windows[g] && R(0, 1)) ? R(1, 40) : 0;   // first positions a window keeps
+    }
     const int slots = R(0, 6);
-    void* c = pa_cache_create(page, groups, pages, windows, slots);
+    void* c = pa_cache_create(page, groups, pages, windows, R(0, 3) ? kept : nullptr, slots);
     const int budget = R(4, 300);
     void* s = pa_sched_create(c, budget, R(0, 1) ? R(1, 100) : 0, R(1, 12), R(0, 1) ? R(50, 2000) : 0, R(0, 1) ? R(1, 200) : 0, R(0, 8), slots > 0 && R(0, 1));
     std::map<long long, int> left;   // new tokens still to come
