@@ -132,9 +132,9 @@ def tedalix_shape(layers=12, width=2048, vocab=65536):
     heads = 16
     mask = dict(size=1024, keep_first=4)
     attention = dict(heads=heads, kv_heads=8, dim=128, vdim=128, scale=128 ** -0.5, mask=mask)
-    parallel = dict(left=dict(heads=heads, kv_heads=4, dim=128, vdim=128, scale=128 ** -0.5, softcap=30.0, mask=dict(size=512)),
-                    right=dict(heads=heads, kv_heads=8, dim=128, vdim=128, conv=4, rank=128), left_scale=0.8, right_scale=0.9)
-    retention = dict(heads=heads, dim=128, vdim=128, rot=dict(base=1000000.0, dims=64),
+    parallel = dict(left=dict(heads=heads, kv_heads=4, dim=128, vdim=128, scale=128 ** -0.5, softcap=50.0, mask=dict(size=512)),
+                    right=dict(heads=heads, kv_heads=8, dim=128, vdim=128, conv=4, rank=128), left_scale=1.0, right_scale=1.0)
+    retention = dict(heads=heads, dim=128, vdim=128, rot=dict(base=10000.0, dims=64),
                      decay=[1.0 - 2.0 ** -(5.0 + 3.0 * h / heads) for h in range(heads)])
     dense = dict(kind="dense", ff=8192)
     out = []

@@ -126,8 +126,8 @@ def _attention_step(ctx, qn, gpu):
 
 MASKED = [  # nh, nkv, hd, vd, page, window, keep_first, softcap, slopes, sink, gate
     (4, 2, 32, 32, 8, 24, 5, 0.0, False, False, False),
-    (4, 1, 64, 64, 16, 96, 6, 0.0, False, False, False),
-    (8, 1, 96, 96, 16, 40, 0, 30.0, True, True, True),
+    (6, 2, 64, 64, 16, 80, 7, 0.0, False, False, False),
+    (4, 2, 96, 96, 16, 48, 0, 25.0, True, True, True),
     (3, 1, 16, 24, 4, 20, 0, 15.0, True, True, True),
     (5, 5, 24, 40, 8, 8, 30, 0.0, False, False, False),
     (6, 3, 128, 128, 16, 64, 0, 5.0, True, True, True),
@@ -199,7 +199,7 @@ def test_attention_under_a_window_with_kept_first_tokens(gpu, dtype, nh, nkv, hd
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("nh,nkv,hd,vd,normed", [(3, 1, 16, 24, True), (8, 1, 96, 96, True), (4, 2, 64, 32, False), (5, 5, 24, 40, True)])
+@pytest.mark.parametrize("nh,nkv,hd,vd,normed", [(3, 1, 16, 24, True), (6, 2, 96, 96, True), (4, 2, 64, 32, False), (5, 5, 24, 40, True)])
 def test_queries_and_keys_normed_over_the_whole_projection(gpu, dtype, nh, nkv, hd, vd, normed):
     """From the merged projection to queries, and keys and values in their pages: one head far larger than the others, so
     that a norm per head would show."""
@@ -232,7 +232,7 @@ def test_queries_and_keys_normed_over_the_whole_projection(gpu, dtype, nh, nkv, 
 
 # ---- the gated delta rule's recurrence alone ---------------------------------------------------------------------------------
 @pytest.mark.parametrize("singles", [False, True])
-@pytest.mark.parametrize("heads,kvh,d,e", [(4, 2, 16, 24), (2, 1, 48, 72), (4, 4, 32, 32), (3, 1, 20, 8), (1, 1, 8, 136), (2, 2, 256, 64),
+@pytest.mark.parametrize("heads,kvh,d,e", [(4, 2, 16, 24), (2, 1, 48, 72), (6, 3, 32, 40), (3, 1, 20, 8), (1, 1, 8, 136), (2, 2, 256, 64),
                                            (8, 4, 128, 128), (2, 1, 100, 40)])
 def test_the_delta_rule_alone(gpu, heads, kvh, d, e, singles):
     """Unequal sequences in one launch, each from a state of its own in a slot of its own: outputs and the states left
