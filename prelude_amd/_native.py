@@ -112,7 +112,7 @@ _KERNEL_API = {
     "pa_attn_masked_mfma_supports": (I, [I, I, I]),
     "pa_qkv_prepare": (I, [P, I, P, c_long, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, F]),
     "pa_delta_prepare": (I, [P, I, P, c_long, I, I, P, I, P, P, P, P, P, c_long, I, P, P, P, P, P, I, I, I, I, I, I]),
-    "pa_gated_delta": (I, [P, P, P, P, P, P, P, P, I, I, I, I, I, I]),
+    "pa_gated_delta": (I, [P, P, P, P, P, P, P, P, I, I, I, I, I]),
     "pa_rotate_halves_f32": (I, [P, I, P, c_long, I, I, I, P, P, P, I, I, I, I, I, F]),
 }
 

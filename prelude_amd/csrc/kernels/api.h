@@ -313,7 +313,7 @@ int pa_delta_prepare(void* stream, int dtype, const void* p, long stride, int of
                      long a_stride, int a_off, const float* a_log, const float* dt_bias, float* out, float* decay, float* beta,
                      int tokens, int nseq, int heads, int kvh, int d, int e);
 int pa_gated_delta(void* stream, const float* x, const float* decay, const float* beta, float* state, const int* state_slots,
-                   const int* cu_q, float* out, int nseq, int heads, int kvh, int d, int e, int portions);
+                   const int* cu_q, float* out, int nseq, int heads, int kvh, int d, int e);
 int pa_rotate_halves_f32(void* stream, int dtype, const void* p, long stride, int q_off, int k_off, int v_off,
                          const float* inv_freq, const int* positions, float* out, int tokens, int heads, int d, int e, int rot,
                          float k_scale);

@@ -90,78 +90,13 @@ __global__ void conv_state_update_kernel(const T* __restrict__ p, size_t stride,
   for (int i = 0; i < keep; ++i) st[i] = fresh[i];
 }
 
-// The recurrence.  A wavefront owns 64 value columns of one (sequence, head); a lane keeps its column of S in
-// registers (D rows, the key width rounded up).  Tokens are walked in order, a block of them staged in LDS.
-// x [T, C] 32-bit as delta_prepare left it ([q | k | v]), decay [T, heads, d], beta [T, heads];
-// state [slots, heads, d, e]; out [T, heads, e].
-template <int D>
-__global__ __launch_bounds__(kWave) void gated_delta_kernel(const float* __restrict__ x, const float* __restrict__ decay,
-                                                           const float* __restrict__ beta, float* __restrict__ state,
-                                                           const int* __restrict__ state_slots, const int* __restrict__ cu_q,
-                                                           float* __restrict__ out, int heads, int kvh, int d, int e) {
-  constexpr int NT = D <= 128 ? 16 : 8;
-  __shared__ float ks[NT][D], qs[NT][D], gs[NT][D];
-  __shared__ float bs[NT];
-  const int seq = blockIdx.x, h = blockIdx.y;
-  const int col = blockIdx.z * kWave + threadIdx.x;
-  const bool live = col < e;
-  const int begin = cu_q[seq], end = cu_q[seq + 1];
-  if (end <= begin) return;
-  const int kh = h / (heads / kvh);
-  const int qk = kvh * d, C = 2 * qk + heads * e;
-  float* S = state + (((size_t)state_slots[seq] * heads + h) * d) * e;
-  float s[D];
-#pragma unroll
-  for (int j = 0; j < D; ++j) s[j] = (live && j < d) ? S[(size_t)j * e + col] : 0.f;
-  for (int t0 = begin; t0 < end; t0 += NT) {
-    const int n = end - t0 < NT ? end - t0 : NT;
-    __syncthreads();
-    for (int i = threadIdx.x; i < n * D; i += kWave) {
-      const int tk = i / D, j = i % D;
-      const size_t t = t0 + tk;
-      const bool in = j < d;
-      qs[tk][j] = in ? x[t * C + kh * d + j] : 0.f;
-      ks[tk][j] = in ? x[t * C + qk + kh * d + j] : 0.f;
-      gs[tk][j] = in ? decay[(t * heads + h) * d + j] : 1.f;
-    }
-    if (threadIdx.x < n) bs[threadIdx.x] = beta[(size_t)(t0 + threadIdx.x) * heads + h];
-    __syncthreads();
-    float v[NT];
-#pragma unroll
-    for (int tk = 0; tk < NT; ++tk) v[tk] = (live && tk < n) ? x[(size_t)(t0 + tk) * C + 2 * qk + h * e + col] : 0.f;
-#pragma unroll
-    for (int tk = 0; tk < NT; ++tk) {
-      if (tk < n) {
-        float kv = 0.f;
-#pragma unroll
-        for (int j = 0; j < D; ++j) {
-          s[j] *= gs[tk][j];
-          kv = fmaf(s[j], ks[tk][j], kv);
-        }
-        const float u = bs[tk] * (v[tk] - kv);
-        float o = 0.f;
-#pragma unroll
-        for (int j = 0; j < D; ++j) {
-          s[j] = fmaf(ks[tk][j], u, s[j]);
-          o = fmaf(s[j], qs[tk][j], o);
-        }
-        if (live) out[((size_t)(t0 + tk) * heads + h) * e + col] = o;
-      }
-    }
-  }
-  if (live) {
-#pragma unroll
-    for (int j = 0; j < D; ++j)
-      if (j < d) S[(size_t)j * e + col] = s[j];
-  }
-}
-
-// The recurrence for portions of prompts: the same sums with a column of S spread over R neighbouring lanes, each
-// keeping D / R rows in registers (four consecutive rows of every R-th group of four, so that the R lanes of a column read
-// one contiguous stretch of LDS), and the two dot products summed across the R lanes inside the wavefront's rows of 16
-// lanes.  A sequence of one head is then 256 / R columns a workgroup instead of 64 a wavefront: sixteen times the
-// wavefronts, and a dependent chain of D / R instead of D multiply-adds a token.  The order of every sum still follows
-// the token's place alone.
+// The recurrence.  x [T, C] 32-bit as delta_prepare left it ([q | k | v]), decay [T, heads, d], beta [T, heads];
+// state [slots, heads, d, e]; out [T, heads, e].  The columns of S do not depend on each other.  A column is spread over
+// R neighbouring lanes, each keeping D / R rows in registers (four consecutive rows of every R-th group of four, so
+// that the R lanes of a column read one contiguous stretch of LDS), and the two dot products are summed across the R
+// lanes inside the wavefront's rows of 16 lanes: a sequence of one head is 256 / R columns a workgroup, and the
+// dependent chain a token D / R multiply-adds.  The order of every sum follows the token's place alone, so outputs
+// and state are the same bits however a prompt is cut into steps.
 template <int R>
 __device__ __forceinline__ float sum_over_lanes(float v) {
   static_assert(R == 8 || R == 16, "a column's lanes lie inside a row of 16");
@@ -386,17 +321,15 @@ extern "C" int pa_delta_prepare(void* stream, int dtype, const void* p, long str
 }
 
 extern "C" int pa_gated_delta(void* stream, const float* x, const float* decay, const float* beta, float* state,
-                              const int* state_slots, const int* cu_q, float* out, int nseq, int heads, int kvh, int d, int e,
-                              int portions) {
+                              const int* state_slots, const int* cu_q, float* out, int nseq, int heads, int kvh, int d, int e) {
   if (nseq == 0) return 0;
   PA_REQUIRE(nseq > 0 && heads > 0 && kvh > 0 && heads % kvh == 0 && d > 0 && e > 0,
              "gated_delta: bad sizes sequences=%d heads=%d key heads=%d d=%d e=%d", nseq, heads, kvh, d, e);
   PA_REQUIRE(d <= 256, "gated_delta: a key width of %d is more than the 256 the kernel takes", d);
   hipStream_t st = (hipStream_t)stream;
-  if (portions) {   // some sequence brings more than a token: a column over several lanes
-    // 16-byte loads of queries, keys and decays where every row of them starts at a multiple of four floats
-    const bool vec = d % 4 == 0 && (2 * kvh * d + heads * e) % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
-                     (reinterpret_cast<uintptr_t>(decay) & 15) == 0;
+  // 16-byte loads of queries, keys and decays where every row of them starts at a multiple of four floats
+  const bool vec = d % 4 == 0 && (2 * kvh * d + heads * e) % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(decay) & 15) == 0;
 #define PA_DELTA_ROWS(D, R)                                                                                                       \
   do {                                                                                                                            \
     dim3 rgrid(nseq, heads, (e + 256 / R - 1) / (256 / R));                                                                       \
@@ -407,21 +340,11 @@ extern "C" int pa_gated_delta(void* stream, const float* x, const float* decay, 
       hipLaunchKernelGGL((gated_delta_rows_kernel<D, R, false>), rgrid, dim3(256), 0, st, x, decay, beta, state, state_slots,      \
                          cu_q, out, heads, kvh, d, e);                                                                            \
   } while (0)
-    if (d <= 32) PA_DELTA_ROWS(32, 8);
-    else if (d <= 64) PA_DELTA_ROWS(64, 16);
-    else if (d <= 128) PA_DELTA_ROWS(128, 16);
-    else PA_DELTA_ROWS(256, 16);
+  if (d <= 32) PA_DELTA_ROWS(32, 8);
+  else if (d <= 64) PA_DELTA_ROWS(64, 16);
+  else if (d <= 128) PA_DELTA_ROWS(128, 16);
+  else PA_DELTA_ROWS(256, 16);
 #undef PA_DELTA_ROWS
-    return check_launch("gated_delta");
-  }
-  dim3 grid(nseq, heads, (e + kWave - 1) / kWave);
-#define PA_DELTA(D) hipLaunchKernelGGL(gated_delta_kernel<D>, grid, dim3(kWave), 0, st, x, decay, beta, state, state_slots, cu_q, \
-                                       out, heads, kvh, d, e)
-  if (d <= 32) PA_DELTA(32);
-  else if (d <= 64) PA_DELTA(64);
-  else if (d <= 128) PA_DELTA(128);
-  else PA_DELTA(256);
-#undef PA_DELTA
   return check_launch("gated_delta");
 }
 

@@ -72,6 +72,117 @@ __global__ __launch_bounds__(kRowThreads) void group_norm_step_kernel(
   }
 }
 
+// Eight consecutive elements of a row as 32-bit values, in 16-byte loads and stores.
+__device__ __forceinline__ void load8(const float* p, float* v) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void load8(const bf16* p, float* v) {
+  const bf16x8 a = *reinterpret_cast<const bf16x8*>(p);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = (float)a[i];
+}
+__device__ __forceinline__ void store8(float* p, const float* v) {
+  *reinterpret_cast<float4*>(p) = float4{v[0], v[1], v[2], v[3]};
+  *reinterpret_cast<float4*>(p + 4) = float4{v[4], v[5], v[6], v[7]};
+}
+__device__ __forceinline__ void store8(bf16* p, const float* v) {
+  bf16x8 a;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) a[i] = (bf16)v[i];
+  *reinterpret_cast<bf16x8*>(p) = a;
+}
+
+// The same step for rows of up to 8 * 256 * VPT elements whose groups are whole pieces of eight: a thread keeps VPT
+// pieces of the row in registers, and everything it will need (the branch, the stream, both weights) is asked for
+// at once.  A wavefront's 64 pieces of one round are 512 consecutive elements; it sums the squares of each group
+// that has pieces among them, and a group's sum is its wavefronts' sums added in their order: one barrier a norm.
+template <typename T, int VPT>
+__global__ __launch_bounds__(256) void group_norm_step_vec_kernel(
+    const T* __restrict__ y, const float* __restrict__ w_add, float* __restrict__ residual,
+    const float* __restrict__ w_out, T* __restrict__ out, const int* __restrict__ rows, int hidden, int groups, float eps) {
+  __shared__ float partial[2][4 * VPT][64];
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const size_t r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : r;
+  const int len = hidden / groups;
+  const int pieces = hidden / 8;
+  float cur[VPT][8], yv[VPT][8], wa[VPT][8], wo[VPT][8];
+  float* res = residual + src * hidden;
+#pragma unroll
+  for (int v = 0; v < VPT; ++v) {
+    const int piece = v * 256 + threadIdx.x;
+    if (piece < pieces) {
+      load8(res + 8 * piece, cur[v]);
+      if (y) {
+        load8(y + r * hidden + 8 * piece, yv[v]);
+        load8(w_add + 8 * piece, wa[v]);
+      }
+      if (out) load8(w_out + 8 * piece, wo[v]);
+    }
+  }
+  // 1 / sqrt(mean^2 + eps) of the group of each of the thread's pieces of `vals`
+  auto group_inv = [&](float (*vals)[8], float* inv, int buf) {
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) {
+      const int piece = v * 256 + threadIdx.x;
+      const bool on = piece < pieces;
+      float ss = 0.f;
+      if (on) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss += vals[v][i] * vals[v][i];
+      }
+      const int e0 = (v * 4 + wave) * 512;          // the wavefront's first element of this round
+      if (e0 < hidden) {
+        const int e1 = (e0 + 512 < hidden ? e0 + 512 : hidden) - 1;
+        const int glo = e0 / len, ghi = e1 / len;
+        const int mine = on ? (8 * piece) / len : -1;
+        for (int g = glo; g <= ghi; ++g) {
+          const float s = wave_sum(mine == g ? ss : 0.f);
+          if (lane == 0) partial[buf][v * 4 + wave][g - glo] = s;
+        }
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) {
+      const int piece = v * 256 + threadIdx.x;
+      inv[v] = 0.f;
+      if (piece < pieces) {
+        const int g = (8 * piece) / len;
+        float total = 0.f;
+        for (int vw = (g * len) / 512; vw <= ((g + 1) * len - 1) / 512; ++vw) total += partial[buf][vw][g - (vw * 512) / len];
+        inv[v] = 1.0f / sqrtf(total / (float)len + eps);
+      }
+    }
+  };
+  float inv[VPT];
+  if (y) {
+    group_inv(yv, inv, 0);
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) {
+      const int piece = v * 256 + threadIdx.x;
+      if (piece < pieces) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) cur[v][i] += yv[v][i] * inv[v] * wa[v][i];
+        store8(res + 8 * piece, cur[v]);
+      }
+    }
+  }
+  if (!out) return;
+  group_inv(cur, inv, 1);
+#pragma unroll
+  for (int v = 0; v < VPT; ++v) {
+    const int piece = v * 256 + threadIdx.x;
+    if (piece < pieces) {
+      float o[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) o[i] = cur[v][i] * inv[v] * wo[v][i];
+      store8(out + r * hidden + 8 * piece, o);
+    }
+  }
+}
+
 // out = a N(z) + b N(z^2) + c N(z^3) + e over a row, z = x (+ bias), powers element by element, N(u) = u over
 // sqrt(mean(u^2) + eps); coeff = (a, b, c, e) on the device.  A workgroup a row; the row is read twice.
 template <typename T>
@@ -199,6 +310,24 @@ extern "C" int pa_group_norm_step(void* stream, int dtype, const void* y, const 
   PA_REQUIRE(!out || w_out, "group_norm_step: an output needs its norm's weight");
   PA_REQUIRE(!(y && rows), "group_norm_step: rows are chosen only where nothing is added");
   hipStream_t st = (hipStream_t)stream;
+  auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  if ((dtype == kF32 || dtype == kBF16) && hidden % 8 == 0 && (hidden / groups) % 8 == 0 && hidden <= 8 * 256 * 4 && aligned(y) &&
+      aligned(w_add) && aligned(residual) && aligned(w_out) && aligned(out)) {
+    const int vpt = (hidden / 8 + 255) / 256;
+#define PA_GNORM(T, V) hipLaunchKernelGGL((group_norm_step_vec_kernel<T, V>), dim3(nrows), dim3(256), 0, st, (const T*)y, w_add, \
+                                          residual, w_out, (T*)out, rows, hidden, groups, eps)
+    if (dtype == kF32) {
+      if (vpt <= 1) PA_GNORM(float, 1);
+      else if (vpt <= 2) PA_GNORM(float, 2);
+      else PA_GNORM(float, 4);
+    } else {
+      if (vpt <= 1) PA_GNORM(bf16, 1);
+      else if (vpt <= 2) PA_GNORM(bf16, 2);
+      else PA_GNORM(bf16, 4);
+    }
+#undef PA_GNORM
+    return check_launch("group_norm_step");
+  }
   const size_t lds = (size_t)hidden * sizeof(float);
   if (dtype == kF32)
     hipLaunchKernelGGL(group_norm_step_kernel<float>, dim3(nrows), dim3(kRowThreads), lds, st, (const float*)y, w_add, residual,

@@ -1768,10 +1768,8 @@ def gated_delta(x: torch.Tensor, decay: torch.Tensor, beta: torch.Tensor, state:
         raise NativeError(f"gated_delta: x {tuple(x.shape)} / decay {tuple(decay.shape)} / beta {tuple(beta.shape)} / state {tuple(state.shape)}")
     out = torch.empty((t, heads, e), dtype=torch.float32, device=x.device)
     if t:
-        # a step of single tokens alone: a lane a column, whole rows of the state read side by side; with portions: a column
-        # over several lanes (the sums are the same up to rounding, in another order)
         check(kernels().pa_gated_delta(_stream(), _ptr(x), _ptr(decay), _ptr(beta), _ptr(state), _ptr(step.state_slots), _ptr(step.cu_q),
-                                       _ptr(out), step.num_seqs, heads, kvh, d, e, int(t > step.num_seqs)))
+                                       _ptr(out), step.num_seqs, heads, kvh, d, e))
     return out
 
 

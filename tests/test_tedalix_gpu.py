@@ -49,7 +49,7 @@ def rnd(shape, seed, dtype, scale=1.0):
 
 # ---- norms in groups, the polynomial activation -----------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("hidden,groups", [(48, 3), (36, 2), (256, 1), (1000, 5), (2048, 4), (4104, 8)])
+@pytest.mark.parametrize("hidden,groups", [(48, 3), (36, 2), (256, 1), (1000, 5), (2048, 4), (4104, 8), (384, 3), (4096, 2), (8192, 4), (1536, 64), (10240, 5)])
 def test_norm_in_groups_around_the_stream(gpu, dtype, hidden, groups):
     from prelude_amd.ops import kernels as K
     eps = 1e-5
@@ -236,9 +236,8 @@ def test_queries_and_keys_normed_over_the_whole_projection(gpu, dtype, nh, nkv, 
                                            (8, 4, 128, 128), (2, 1, 100, 40)])
 def test_the_delta_rule_alone(gpu, heads, kvh, d, e, singles):
     """Unequal sequences in one launch, each from a state of its own in a slot of its own: outputs and the states left
-    behind, for steps with portions (a column of the state over several lanes) and steps of single tokens alone (a lane
-    a column).  A key written once with beta 1 and no decay is read back by the same query, overwritten by the next
-    writes under the same key."""
+    behind, for steps with portions and steps of single tokens alone.  A key written once with beta 1 and no decay is
+    read back by the same query, and so are the next writes under the same key."""
     from prelude_amd.ops import kernels as K
     lengths = [1, 1, 1] if singles else [1, 47, 16, 17, 2, 33]
     slots = [4, 0, 6] if singles else [7, 2, 5, 0, 4, 1]
