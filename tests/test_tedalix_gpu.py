@@ -388,6 +388,43 @@ def test_what_a_position_sees_ends_at_the_edges_of_its_mask(gpu, kind, window, k
         check(last(other(j)), want, "float32", f"token {j} is inside what {i} sees")
 
 
+@pytest.mark.parametrize("decoded", [False, True])
+@pytest.mark.parametrize("kind,window,keep", [("attention", 40, 5), ("attention", 33, 0), ("attention", 20, 37), ("parallel", 48, 0)])
+def test_the_edges_of_the_mask_on_the_matrix_cores(gpu, kind, window, keep, decoded):
+    """The same with heads of 64 under the bfloat16 engine, where attention runs on the matrix cores: a changed token
+    just outside the mask leaves the logits bit for bit as they are (the same instructions on the same numbers); one
+    just inside moves them as far as it moves the plain logits."""
+    if kind == "attention":
+        cfg = one_layer(kind, **{"mask": {"size": window, "keep_first": keep}, "dim": 64, "vdim": 64, "scale": 0.125})
+    else:
+        cfg = one_layer(kind, **{"left.mask": {"size": window}, "left.dim": 64, "left.vdim": 64, "left.scale": 0.125, "right_scale": 0.0})
+    w = pt.random_weights(cfg, 62)
+    path = write_model(cfg, w)
+    n = 2 * window + keep + 70                 # more than a tile of 64 tokens behind the kept ones
+    toks = torch.randint(0, cfg["vocab"], (n,), generator=torch.Generator().manual_seed(63)).tolist()
+    i = n - 1
+    cuts = [n - 19] if decoded else [n]
+
+    def last(t):
+        return run_cut(path, "bfloat16", t, cuts, page=16)[-1]
+
+    def other(j):
+        t = list(toks)
+        t[j] = (t[j] + 1 + j) % cfg["vocab"]
+        return t
+    base = last(toks)
+    ref = pt.forward(cfg, w, toks)
+    mostly(base[None], ref[-1:], "bfloat16", "as it is")
+    outside = [j for j in (i - window, i - window - 1) if j >= keep] + ([keep] if keep and keep < i - window + 1 else [])
+    inside = [i - window + 1] + ([keep - 1] if keep else [])
+    for j in outside:
+        assert np.array_equal(last(other(j)), base), f"token {j} is outside what {i} sees"
+    for j in inside:
+        moved = float((pt.forward(cfg, w, other(j))[-1] - ref[-1]).abs().max())
+        got = float(np.abs(last(other(j)) - base).max())
+        assert got > 0 and abs(got - moved) <= 0.5 * moved + 0.02 * float(ref.std()), f"token {j} is inside what {i} sees: {got} against {moved}"
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_a_sink_takes_weight_at_the_first_token(gpu, dtype):
     """A sink far above the scores: the attention half all but vanishes, also at the first token, where a softmax
