@@ -25,7 +25,7 @@
 // matrix cores (`attn_masked_mfma_kernel` below), with the inner step of the plain matrix-core kernels: a wavefront
 // owns 16 tokens of two heads that share a KV head (one when the group is odd) and walks, 32 keys a step, first the steps that hold kept
 // first tokens and then the window's; a sequence that brings one token has its steps dealt out to the workgroup's
-// four wavefronts, whose sums are merged through LDS.
+// wavefronts (eight where the whole step is single tokens), whose sums are merged through LDS.
 #include "common.h"
 #include "api.h"
 #include "attention_mfma_core.h"
@@ -245,13 +245,14 @@ struct MaskedArgs {
   float out_scale;
 };
 
-// Grid (tiles of 64 tokens, nkv * head groups, sequences); four wavefronts.
-template <int KD, int VD, int GT>
-__global__ __launch_bounds__(256, 2) void attn_masked_mfma_kernel(MaskedArgs a) {
+// Grid (tiles of 64 tokens, nkv * head groups, sequences); WAVES wavefronts: four, or eight for steps in which every
+// sequence brings one token (half the steps a wavefront, which is what such a step's time is made of).
+template <int KD, int VD, int GT, int WAVES>
+__global__ __launch_bounds__(WAVES* kWave, WAVES == 8 ? 1 : 2) void attn_masked_mfma_kernel(MaskedArgs a) {
   constexpr int OT = VD / 16;
   constexpr int KS = KD / 32;
-  __shared__ float lds_o[4][GT][VD];
-  __shared__ float lds_ml[4][GT][2];
+  __shared__ float lds_o[WAVES][GT][VD];
+  __shared__ float lds_ml[WAVES][GT][2];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int g = lane / 16, r = lane % 16;
   const int group = a.nh / a.nkv;
@@ -263,7 +264,8 @@ __global__ __launch_bounds__(256, 2) void attn_masked_mfma_kernel(MaskedArgs a) 
   const int q_len = a.cu_q[seq + 1] - row0;
   if (q_len <= 0) return;
   const int ctx = a.context_lens[seq];
-  const bool single = q_len == 1;            // one token: its steps are dealt out to the four wavefronts
+  const bool single = q_len == 1;            // one token: its steps are dealt out to the wavefronts
+  if (WAVES != 4 && !single) return;         // (the launch with more wavefronts is for steps of single tokens alone)
   const int tiles = (q_len + 63) / 64;
   const int tile = tiles - 1 - (int)blockIdx.x;   // late tiles first
   if (tile < 0) return;
@@ -329,7 +331,7 @@ __global__ __launch_bounds__(256, 2) void attn_masked_mfma_kernel(MaskedArgs a) 
     }
     return;
   }
-  for (int i = wave; i < n_steps; i += 4) {
+  for (int i = wave; i < n_steps; i += WAVES) {
     const int key0 = key_of(i);
     KFrag<KD> kf;
     load_k_gap<KD>(w, kept, key0, g, r, kf);
@@ -353,10 +355,10 @@ __global__ __launch_bounds__(256, 2) void attn_masked_mfma_kernel(MaskedArgs a) 
     const int j = e / VD, d = e % VD;
     float mm = lds_ml[0][j][0];
 #pragma unroll
-    for (int v = 1; v < 4; ++v) mm = fmaxf(mm, lds_ml[v][j][0]);
+    for (int v = 1; v < WAVES; ++v) mm = fmaxf(mm, lds_ml[v][j][0]);
     float o = 0.f, l = 0.f;
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {   // in the order of the wavefronts
+    for (int v = 0; v < WAVES; ++v) {   // in the order of the wavefronts
       const float f = lds_ml[v][j][0] == -INFINITY ? 0.f : exp2f(lds_ml[v][j][0] - mm);
       o += lds_o[v][j][d] * f;
       l += lds_ml[v][j][1] * f;
@@ -452,7 +454,12 @@ extern "C" int pa_attn_masked(void* stream, int dtype, const void* q, const void
                  score_map(scale, softcap, sink), softcap > 0.f ? 1.0f : 1.0f / scale, slopes, (const bf16*)gate,
                  (size_t)gate_stride, out_scale};
     dim3 mgrid((max_q_len + 63) / 64, nkv * (group / gt), nseq);
-#define PA_MASKED(D, GT) hipLaunchKernelGGL((attn_masked_mfma_kernel<D, D, GT>), mgrid, dim3(256), 0, st, a)
+    const bool singles = max_q_len == 1;
+#define PA_MASKED(D, GT)                                                                                      \
+  do {                                                                                                        \
+    if (singles) hipLaunchKernelGGL((attn_masked_mfma_kernel<D, D, GT, 8>), mgrid, dim3(512), 0, st, a);       \
+    else hipLaunchKernelGGL((attn_masked_mfma_kernel<D, D, GT, 4>), mgrid, dim3(256), 0, st, a);               \
+  } while (0)
 #define PA_MASKED_GT(D)              \
   do {                               \
     if (gt == 2) PA_MASKED(D, 2);    \
