@@ -201,6 +201,7 @@ __global__ __launch_bounds__(256) void gated_delta_rows_kernel(const float* __re
   for (int t0 = begin; t0 < end; t0 += NT, buf ^= 1) {
     const bool more = t0 + NT < end;
     if (more) fetch(t0 + NT);
+    float ob[NT];
 #pragma unroll
     for (int tk = 0; tk < NT; ++tk) {
       float4 kk[NV];
@@ -228,8 +229,14 @@ __global__ __launch_bounds__(256) void gated_delta_rows_kernel(const float* __re
         po[2] = fmaf(s[i][2], qq.z, po[2]);
         po[3] = fmaf(s[i][3], qq.w, po[3]);
       }
-      const float o = sum_over_lanes<R>((po[0] + po[1]) + (po[2] + po[3]));
-      if (live && rho == 0 && t0 + tk < end) out[((size_t)(t0 + tk) * heads + h) * e + col] = o;
+      ob[tk] = sum_over_lanes<R>((po[0] + po[1]) + (po[2] + po[3]));
+    }
+    // the block's outputs leave together: a store a token would end a basic block a token, and the reads of the next
+    // token's rows could not be moved ahead of this token's sums
+    if (live && rho == 0) {
+#pragma unroll
+      for (int tk = 0; tk < NT; ++tk)
+        if (t0 + tk < end) out[((size_t)(t0 + tk) * heads + h) * e + col] = ob[tk];
     }
     if (more) {
       put(buf ^ 1);
