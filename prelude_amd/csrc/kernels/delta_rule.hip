@@ -17,28 +17,43 @@ namespace pa {
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
 __device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
-// A workgroup a token.  p [T, stride] holds, from column `off`, the channels [qk | qk | vv] (queries and keys of
-// `kvh` heads of d, values of `heads` heads of e).  Every channel c: y_t = silu(sum_s w[c, s] x_(t - (taps - 1 - s))),
-// inputs before the step's first token of the sequence from conv_state [slots, C, taps - 1] (oldest first; zero for
-// a request that starts).  Then queries and keys become unit vectors per head (x / sqrt(sum x^2 + 1e-6)), the
-// queries also times d^(-1/2).  out [T, C] 32-bit.  Also: decay [T, heads * d] = exp(-exp(a_log[h]) *
-// softplus(a[t, h * d + j] + dt_bias[h * d + j])) from a [T, a_stride] at column a_off, and beta [T, heads] =
-// sigmoid(b[t, h]) from p at column b_off.
+// A workgroup of two wavefronts a (token, unit).  p [T, stride] holds, from column `off`, the channels [qk | qk | vv]
+// (queries and keys of `kvh` heads of d, values of `heads` heads of e).  Every channel c:
+// y_t = silu(sum_s w[c, s] x_(t - (taps - 1 - s))), inputs before the step's first token of the sequence from
+// conv_state [slots, C, taps - 1] (oldest first; zero for a request that starts).  The units, blockIdx.y: a query or
+// key head (2 kvh of them), whose d channels then become a unit vector (x / sqrt(sum x^2 + 1e-6)), a query also times
+// d^(-1/2); a value head's e channels; a head's d decays, decay [T, heads * d] = exp(-exp(a_log[h]) *
+// softplus(a[t, h * d + j] + dt_bias[h * d + j])) from a [T, a_stride] at column a_off, the first of them also
+// beta [T, heads] = sigmoid(b[t, h]) from p at column b_off.  out [T, C] 32-bit.
+constexpr int kPrepareThreads = 128;
+constexpr int kPrepareMost = 256;   // most channels of a query or key head
+
 template <typename T>
-__global__ __launch_bounds__(256) void delta_prepare_kernel(
+__global__ __launch_bounds__(kPrepareThreads) void delta_prepare_kernel(
     const T* __restrict__ p, size_t stride, int off, int b_off, const float* __restrict__ w, int taps,
     const float* __restrict__ conv_state, const int* __restrict__ seq_of_token, const int* __restrict__ cu_q,
     const int* __restrict__ state_slots, const T* __restrict__ a, size_t a_stride, int a_off,
     const float* __restrict__ a_log, const float* __restrict__ dt_bias, float* __restrict__ out,
     float* __restrict__ decay, float* __restrict__ beta, int heads, int kvh, int d, int e) {
-  extern __shared__ float y[];
-  const int t = blockIdx.x;
+  __shared__ float sums[kPrepareThreads / kWave];
+  const int t = blockIdx.x, u = blockIdx.y;
+  const int qk = kvh * d, C = 2 * qk + heads * e;
+  if (u >= 2 * kvh + heads) {                 // a head's decays
+    const int h = u - 2 * kvh - heads;
+    const float rate = expf(a_log[h]);
+    for (int j = threadIdx.x; j < d; j += kPrepareThreads) {
+      const int i = h * d + j;
+      decay[(size_t)t * heads * d + i] = expf(-rate * softplus_f(to_f32(a[(size_t)t * a_stride + a_off + i]) + dt_bias[i]));
+    }
+    if (h == 0)
+      for (int g = threadIdx.x; g < heads; g += kPrepareThreads)
+        beta[(size_t)t * heads + g] = 1.0f / (1.0f + expf(-to_f32(p[(size_t)t * stride + b_off + g])));
+    return;
+  }
   const int seq = seq_of_token[t];
   const int local = t - cu_q[seq];          // tokens of this sequence in the step before this one
-  const int slot = state_slots[seq];
-  const int qk = kvh * d, C = 2 * qk + heads * e;
-  const float* st = conv_state + (size_t)slot * C * (taps - 1);
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+  const float* st = conv_state + (size_t)state_slots[seq] * C * (taps - 1);
+  auto conv = [&](int c) {
     float acc = 0.f;
     for (int s = 0; s < taps; ++s) {
       const int back = taps - 1 - s;          // how many tokens back this tap reaches
@@ -47,26 +62,33 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(
       else x = st[(size_t)c * (taps - 1) + (taps - 1) - (back - local)];
       acc = fmaf(w[(size_t)c * taps + s], x, acc);
     }
-    y[c] = silu_f(acc);
+    return silu_f(acc);
+  };
+  if (u >= 2 * kvh) {                         // a value head
+    const int c0 = 2 * qk + (u - 2 * kvh) * e;
+    for (int j = threadIdx.x; j < e; j += kPrepareThreads) out[(size_t)t * C + c0 + j] = conv(c0 + j);
+    return;
   }
+  const int c0 = u * d;                       // a query or key head: a unit vector
+  float y[kPrepareMost / kPrepareThreads];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < kPrepareMost / kPrepareThreads; ++i) {
+    const int j = i * kPrepareThreads + threadIdx.x;
+    y[i] = j < d ? conv(c0 + j) : 0.f;
+    ss += y[i] * y[i];
+  }
+  ss = wave_sum(ss);
+  if (threadIdx.x % kWave == 0) sums[threadIdx.x / kWave] = ss;
   __syncthreads();
-  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave, nwaves = blockDim.x / kWave;
-  for (int v = wave; v < 2 * kvh; v += nwaves) {      // vectors to bring to unit length: kvh of q, then kvh of k
-    float ss = 0.f;
-    for (int j = lane; j < d; j += kWave) ss += y[v * d + j] * y[v * d + j];
-    ss = wave_sum(ss);
-    float f = 1.0f / sqrtf(ss + 1e-6f);
-    if (v < kvh) f *= 1.0f / sqrtf((float)d);
-    for (int j = lane; j < d; j += kWave) y[v * d + j] *= f;
+  ss = sums[0] + sums[1];
+  float f = 1.0f / sqrtf(ss + 1e-6f);
+  if (u < kvh) f *= 1.0f / sqrtf((float)d);
+#pragma unroll
+  for (int i = 0; i < kPrepareMost / kPrepareThreads; ++i) {
+    const int j = i * kPrepareThreads + threadIdx.x;
+    if (j < d) out[(size_t)t * C + c0 + j] = y[i] * f;
   }
-  __syncthreads();
-  for (int c = threadIdx.x; c < C; c += blockDim.x) out[(size_t)t * C + c] = y[c];
-  for (int i = threadIdx.x; i < heads * d; i += blockDim.x) {
-    const float rate = expf(a_log[i / d]);
-    decay[(size_t)t * heads * d + i] = expf(-rate * softplus_f(to_f32(a[(size_t)t * a_stride + a_off + i]) + dt_bias[i]));
-  }
-  for (int h = threadIdx.x; h < heads; h += blockDim.x)
-    beta[(size_t)t * heads + h] = 1.0f / (1.0f + expf(-to_f32(p[(size_t)t * stride + b_off + h])));
 }
 
 // After the step's convolutions: a sequence's carried inputs become the last taps - 1 inputs it has seen.  A thread a
@@ -302,20 +324,20 @@ extern "C" int pa_delta_prepare(void* stream, int dtype, const void* p, long str
              "delta_prepare: bad sizes tokens=%d sequences=%d heads=%d key heads=%d d=%d e=%d", tokens, nseq, heads, kvh, d, e);
   PA_REQUIRE(taps >= 1 && taps <= 9, "delta_prepare: a convolution of %d taps is outside 1..9", taps);
   const long C = 2L * kvh * d + (long)heads * e;
-  PA_REQUIRE(C <= 15360, "delta_prepare: %ld channels are more than the 15360 the kernel takes", C);
   PA_REQUIRE(off >= 0 && off + C <= stride && b_off >= 0 && b_off + heads <= stride && a_off >= 0 &&
              a_off + (long)heads * d <= a_stride, "delta_prepare: the columns do not fit their rows");
   hipStream_t st = (hipStream_t)stream;
-  const size_t lds = (size_t)C * sizeof(float);
+  PA_REQUIRE(d <= kPrepareMost, "delta_prepare: a key width of %d is more than the %d the kernel takes", d, kPrepareMost);
+  const dim3 pgrid(tokens, 2 * kvh + 2 * heads);
   if (dtype == kF32) {
-    hipLaunchKernelGGL(delta_prepare_kernel<float>, dim3(tokens), dim3(256), lds, st, (const float*)p, (size_t)stride, off,
+    hipLaunchKernelGGL(delta_prepare_kernel<float>, pgrid, dim3(kPrepareThreads), 0, st, (const float*)p, (size_t)stride, off,
                        b_off, w, taps, conv_state, seq_of_token, cu_q, state_slots, (const float*)a, (size_t)a_stride, a_off,
                        a_log, dt_bias, out, decay, beta, heads, kvh, d, e);
     if (taps > 1)
       hipLaunchKernelGGL(conv_state_update_kernel<float>, dim3((unsigned)((C + 255) / 256), nseq), dim3(256), 0, st,
                          (const float*)p, (size_t)stride, off, (int)C, taps, conv_state, cu_q, state_slots, nseq);
   } else if (dtype == kBF16) {
-    hipLaunchKernelGGL(delta_prepare_kernel<bf16>, dim3(tokens), dim3(256), lds, st, (const bf16*)p, (size_t)stride, off, b_off,
+    hipLaunchKernelGGL(delta_prepare_kernel<bf16>, pgrid, dim3(kPrepareThreads), 0, st, (const bf16*)p, (size_t)stride, off, b_off,
                        w, taps, conv_state, seq_of_token, cu_q, state_slots, (const bf16*)a, (size_t)a_stride, a_off, a_log,
                        dt_bias, out, decay, beta, heads, kvh, d, e);
     if (taps > 1)
