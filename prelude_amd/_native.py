@@ -72,7 +72,7 @@ _KERNEL_API = {
     "pa_rmsnorm_wide": (I, [P, I, P, P, I, c_long, P, P, P, P, I, I, F]),
     "pa_clamped_gate": (I, [P, I, P, P, I, I, F, F]),
     "pa_relu_squared": (I, [P, I, P, P, c_long]),
-    "pa_latent_prep": (I, [P, I, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F]),
+    "pa_latent_prep": (I, [P, I, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, c_long]),
     "pa_rotate_pairs": (I, [P, I, P, P, P, P, I, I, I, I, I, I, I, I]),
     "pa_head_linear": (I, [P, I, P, P, P, I, I, I, I, c_long, c_long, c_long, c_long]),
     "pa_latent_attn": (I, [P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F]),
@@ -86,8 +86,8 @@ _KERNEL_API = {
     "pa_head_linear_mfma": (I, [P, P, P, P, I, I, I, I, c_long, c_long, c_long, c_long]),
     "pa_moe_combine": (I, [P, I, P, P, P, F, P, P, P, I, I, I]),
     "pa_gemm_narrow": (I, [P, P, P, P, I, I, I, c_long, c_long]),
-    "pa_moe_route": (I, [P, P, I, P, P, P, P, I, I, I, F, I]),
-    "pa_qknorm_rope_kv_freq": (I, [P, I, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I]),
+    "pa_moe_route": (I, [P, P, I, P, P, P, P, I, I, I, F, I, P, I]),
+    "pa_qknorm_rope_kv_freq": (I, [P, I, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, P]),
     "pa_attn_decode_sink": (I, [P, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, F, P, I, I]),
     "pa_attn_prefill_sink": (I, [P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, P]),
     "pa_attn_generic_sink": (I, [P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, F, P]),
@@ -108,12 +108,20 @@ _KERNEL_API = {
     "pa_group_norm_step": (I, [P, I, P, P, P, P, P, P, I, I, I, F]),
     "pa_poly_norm": (I, [P, I, P, P, P, P, I, I, F]),
     "pa_head_norm_gate": (I, [P, I, P, P, c_long, P, P, c_long, I, I, I, F, I, F]),
-    "pa_attn_masked": (I, [P, I, P, P, P, P, I, P, P, P, c_long, I, I, I, I, I, I, I, I, F, F, P, P, P, c_long, F, P, P, I, I]),
+    "pa_attn_masked": (I, [P, I, P, P, P, P, I, P, P, P, c_long, I, I, I, I, I, I, I, I, F, F, P, P, P, c_long, F, P, P, I, I, I]),
     "pa_attn_masked_mfma_supports": (I, [I, I, I]),
     "pa_qkv_prepare": (I, [P, I, P, c_long, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, F]),
     "pa_delta_prepare": (I, [P, I, P, c_long, I, I, P, I, P, P, P, P, P, c_long, I, P, P, P, P, P, I, I, I, I, I, I]),
     "pa_gated_delta": (I, [P, P, P, P, P, P, P, P, I, I, I, I, I]),
     "pa_rotate_halves_f32": (I, [P, I, P, c_long, I, I, I, P, P, P, I, I, I, I, I, F]),
+    "pa_pair_embed": (I, [P, I, P, P, P, P, P, P, P, P, P, I, I, I, I, c_long, c_long, F]),
+    "pa_time_conv_add": (I, [P, I, P, P, P, P, P, P, P, I, I, I, I]),
+    "pa_stream_add_row": (I, [P, P, P, I, I]),
+    "pa_stream_add_branches": (I, [P, I, P, P, P, c_long]),
+    "pa_qkv_rope_prepare": (I, [P, I, P, c_long, I, I, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I]),
+    "pa_diff_combine": (I, [P, I, P, P, I, I, I, F, F, F]),
+    "pa_sigmoid_gate": (I, [P, I, P, c_long, P, c_long, P, I, I]),
+    "pa_cap_logits": (I, [P, P, c_long, F]),
 }
 
 _HOST_API = {

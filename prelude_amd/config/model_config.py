@@ -629,3 +629,157 @@ class TedalixConfig:
             raise ConfigError(f"failed to parse {a} config: `norm.groups` ({groups}) does not divide `width` ({width})")
         return cls(vocab=_positive(raw, "vocab", int, a, ""), width=width, norm_eps=_positive(norm, "eps", float, a, "norm."),
                    norm_groups=groups, layers=tuple(layers))
+
+
+# ---------------------------------------------------------------------------
+@dataclasses.dataclass(frozen=True)
+class NivasunMixerConfig:
+    heads: int
+    kv_heads: int       # latent attention: as many as heads (every head has keys of its own, from the latent)
+    dim: int
+    vdim: int
+    scale: float
+    window: int         # the query at i sees the key at j with 0 <= i - j < window
+    rot_dims: int = 0   # the first dimensions of a head (of a map) that turn; 0: none
+    rot_base: float = 0.0
+    kv_rank: int = 0    # latent attention
+    q_rank: int = 0
+    diff: float = 0.0   # differential attention
+
+
+@dataclasses.dataclass(frozen=True)
+class NivasunMlpConfig:
+    ff: int
+    experts: int
+    top: int
+    shared_ff: int      # 0: no shared expert
+
+
+@dataclasses.dataclass(frozen=True)
+class NivasunLayerConfig:
+    type: str
+    mixer: NivasunMixerConfig
+    mlp: Optional[NivasunMlpConfig]
+
+
+@dataclasses.dataclass(frozen=True)
+class NivasunConfig:
+    """Nivasun: a decoder whose layers are listed one by one in ``layers``; a stretch of them (``loop``) runs several
+    times in a row on the same tensors.  A layer has one norm (a single number as its weight) whose output the mixer
+    reads through a short convolution over time and the feed-forward as it is; both are added to the stream together.
+    Mixers: ``attention`` (the keys are the values, rotation in halves, a temperature and a sink per head),
+    ``latent_attention`` (queries, keys and values through latents, a gate on the output), ``attention_2`` (two maps a
+    head, one taken off the other), all under a sliding window.  The feed-forward is routed experts with a gated shared
+    one, or absent.  The embedding adds a row chosen by the token and the one before it; the logits are capped.  Every
+    size and constant is read from here; there is no longest position and no end-of-sequence id."""
+    vocab: int
+    width: int
+    norm_eps: float
+    taps: int
+    embed_scale: float
+    buckets: int
+    mul_prev: int
+    mul_cur: int
+    logit_cap: float            # 0: none
+    loop_start: int
+    loop_stop: int
+    loop_times: int             # 1 with start == stop: no loop
+    layers: Tuple[NivasunLayerConfig, ...]
+
+    ARCH = "Nivasun"
+    MIXERS = ("attention", "latent_attention", "attention_2")
+
+    @classmethod
+    def _rot(cls, m: Mapping[str, Any], mw: str, dim: int):
+        a = cls.ARCH
+        rot = _obj(m, "rot", a, mw, optional=True)
+        if rot is None:
+            return 0, 0.0
+        dims = _get(rot, "dims", int, a, default=0)
+        if dims % 2 or dims > dim:
+            raise ConfigError(f"failed to parse {a} config: `{mw}rot.dims` ({dims}) must be even and at most `dim` ({dim})")
+        return dims, (_positive(rot, "base", float, a, mw + "rot.") if dims else 0.0)
+
+    @classmethod
+    def _mixer(cls, kind: str, m: Mapping[str, Any], mw: str) -> NivasunMixerConfig:
+        a = cls.ARCH
+        heads = _positive(m, "heads", int, a, mw)
+        dim = _positive(m, "dim", int, a, mw)
+        scale = _positive(m, "scale", float, a, mw)
+        window = _positive(_obj(m, "mask", a, mw), "size", int, a, mw + "mask.")
+        if kind == "latent_attention":
+            return NivasunMixerConfig(heads, heads, dim, _positive(m, "vdim", int, a, mw), scale, window,
+                                      kv_rank=_positive(m, "kv_rank", int, a, mw), q_rank=_positive(m, "q_rank", int, a, mw))
+        kv_heads = _positive(m, "kv_heads", int, a, mw)
+        if heads % kv_heads:
+            raise ConfigError(f"failed to parse {a} config: `{mw}heads` ({heads}) is no multiple of `kv_heads` ({kv_heads})")
+        dims, base = cls._rot(m, mw, dim)
+        if kind == "attention":
+            # the values are the keys, so their size is the keys' and may go unsaid
+            vdim = _positive(m, "vdim", int, a, mw) if m.get("vdim") is not None else dim
+            if vdim != dim:
+                raise ConfigError(f"failed to parse {a} config: `{mw}vdim` ({vdim}) must equal `dim` ({dim}): the values are the keys")
+            return NivasunMixerConfig(heads, kv_heads, dim, dim, scale, window, dims, base)
+        diff = _get(m, "diff", float, a)
+        return NivasunMixerConfig(heads, kv_heads, dim, _positive(m, "vdim", int, a, mw), scale, window, dims, base, diff=diff)
+
+    @classmethod
+    def _mlp(cls, f: Optional[Mapping[str, Any]], fw: str) -> Optional[NivasunMlpConfig]:
+        a = cls.ARCH
+        if f is None:
+            return None
+        fk = _get(f, "kind", str, a, default="moe")
+        if fk != "moe":
+            raise ConfigError(f"failed to parse {a} config: `{fw}kind` {fk!r} is not one of ['moe']")
+        router = _obj(f, "router", a, fw)
+        shared = _obj(f, "shared", a, fw, optional=True)
+        mlp = NivasunMlpConfig(ff=_positive(_obj(f, "expert", a, fw), "ff", int, a, fw + "expert."),
+                               experts=_positive(router, "experts", int, a, fw + "router."),
+                               top=_positive(router, "top", int, a, fw + "router."),
+                               shared_ff=_positive(shared, "ff", int, a, fw + "shared.") if shared is not None else 0)
+        if mlp.top > mlp.experts:
+            raise ConfigError(f"failed to parse {a} config: `{fw}router.top` ({mlp.top}) exceeds `router.experts` ({mlp.experts})")
+        return mlp
+
+    @classmethod
+    def from_dict(cls, raw: Mapping[str, Any]) -> "NivasunConfig":
+        a = cls.ARCH
+        layers_raw = raw.get("layers")
+        if not isinstance(layers_raw, list) or not layers_raw:
+            raise ConfigError(f"failed to parse {a} config: `layers` must be a non-empty list")
+        layers = []
+        for i, lr in enumerate(layers_raw):
+            w = f"layers[{i}]."
+            if not isinstance(lr, dict):
+                raise ConfigError(f"failed to parse {a} config: `layers[{i}]` must be an object")
+            kind = _get(lr, "type", str, a)
+            if kind not in cls.MIXERS:
+                raise ConfigError(f"failed to parse {a} config: `{w}type` {kind!r} is not one of {list(cls.MIXERS)}")
+            layers.append(NivasunLayerConfig(kind, cls._mixer(kind, _obj(lr, "mixer", a, w), w + "mixer."),
+                                             cls._mlp(_obj(lr, "mlp", a, w, optional=True), w + "mlp.")))
+        n = len(layers)
+        loop = _obj(raw, "loop", a, optional=True)
+        start, stop, times = 0, 0, 1
+        if loop is not None:
+            start, stop = _get(loop, "start", int, a), _get(loop, "stop", int, a)
+            times = _positive(loop, "times", int, a, "loop.")
+            if not 0 <= start <= stop <= n:
+                raise ConfigError(f"failed to parse {a} config: `loop.start` ({start}) and `loop.stop` ({stop}) must lie in "
+                                  f"order within the {n} layers")
+        emb = _obj(raw, "embedding", a)
+        pair = _obj(emb, "bigram", a, "embedding.")
+        pw = "embedding.bigram."
+        for key in ("mul_prev", "mul_cur"):
+            try:
+                _get(pair, key, int, a)
+            except ConfigError as e:
+                raise ConfigError(str(e).replace(f"`{key}`", f"`{pw}{key}`")) from None
+        cap = _get(raw, "logit_softcap", float, a, default=0.0)
+        if cap < 0:
+            raise ConfigError(f"failed to parse {a} config: `logit_softcap` must not be negative, got {cap!r}")
+        return cls(vocab=_positive(raw, "vocab", int, a, ""), width=_positive(raw, "width", int, a, ""),
+                   norm_eps=_positive(_obj(raw, "norm", a), "eps", float, a, "norm."),
+                   taps=_positive(_obj(raw, "canon", a), "taps", int, a, "canon."),
+                   embed_scale=_get(emb, "scale", float, a, default=1.0), buckets=_positive(pair, "buckets", int, a, pw),
+                   mul_prev=_get(pair, "mul_prev", int, a), mul_cur=_get(pair, "mul_cur", int, a), logit_cap=cap,
+                   loop_start=start, loop_stop=stop, loop_times=times, layers=tuple(layers))

@@ -49,11 +49,12 @@ int pa_qknorm_rope_kv(void* stream, int dtype, const void* qkv, const float* q_w
 
 // pa_qknorm_rope_kv from the rotary frequencies alone (inv_freq [rot / 2], the angle position * inv_freq[j] taken in
 // 32-bit in the kernel: no tables, no longest position); v_from_k: qkv is [tokens, (nh + nkv) * hd] and the cached
-// value of a head is its key as projected, before norm and rotation.
+// value of a head is its key as projected, before norm and rotation.  q_scale (or null) [nh]: every query head times
+// its number, in 32-bit before it is rounded (a temperature per head).
 int pa_qknorm_rope_kv_freq(void* stream, int dtype, const void* qkv, const float* q_weight, const float* k_weight,
                            const float* inv_freq, const int* positions, const int* slots, void* q_out, void* k_cache,
                            void* v_cache, int tokens, int nh, int nkv, int hd, int rot, int page_size, float eps,
-                           int v_from_k);
+                           int v_from_k, const float* q_scale);
 
 // C[m, n] = X[m, k] W[n, k]^T, bfloat16 with 32-bit accumulation, by hipBLASLt called directly; `workspace` is
 // device memory its kernels may use.  The first call with a shape makes and keeps that shape's plan in host memory.
@@ -234,7 +235,7 @@ int pa_lightning_attn_chunked(void* stream, int dtype, const void* qkv, long ld,
 // [pages, rank, page_size], the normed latent once more with the token's offset in its page running fastest.
 int pa_latent_prep(void* stream, int dtype, const void* in, const float* wq, const float* wc, const float* inv_freq,
                    const int* positions, const int* slots, void* cq_out, void* cache, void* cache_t, int page_size,
-                   int tokens, int q_rank, int rank, int rot, int rot_dims, float eps);
+                   int tokens, int q_rank, int rank, int rot, int rot_dims, float eps, long in_stride);
 // in [tokens, heads, in_stride] -> out [tokens, heads, out_stride]: `width` elements from in_off to out_off of every
 // head, the first rot_dims of them rotated in pairs
 int pa_rotate_pairs(void* stream, int dtype, const void* in, void* out, const float* inv_freq, const int* positions,
@@ -271,12 +272,15 @@ int pa_moe_combine(void* stream, int dtype, const float* y, const int* place, co
 // largest s + correction[e] (correction null: none) -> choice [tokens, top]; weights [tokens, top] = their s over the
 // sum of the chosen s (+ 1e-20), times scale.  gate_out (or null) [tokens] = sigmoid(logits[t, gate_col]), a gate a
 // token for a shared expert, from one more column of the same product.
+// bias (or null) [experts] is added to the logits first.  by_logit: the choice goes by the logits themselves (+ bias; no
+// correction) and the weights are the softmax over the chosen logits alone, times scale.
 int pa_moe_route(void* stream, const float* logits, int ld, const float* correction, int* choice, float* weights,
-                 float* gate_out, int tokens, int experts, int top, float scale, int gate_col);
+                 float* gate_out, int tokens, int experts, int top, float scale, int gate_col, const float* bias, int by_logit);
 // The same two products on the matrix cores (grouped_mfma.hip; bfloat16 operands, K a multiple of 8): the weight as
 // stored, [group, N, K].
 // act 2 (here only): the weight's rows alternate gate_j, up_j and y [entries, N / 2] receives the clamped gated pair
-// g * sigmoid(alpha g) * (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit).
+// g * sigmoid(alpha g) * (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit).  act 3: the same rows, the
+// plain gated pair silu(gate) * up.
 int pa_moe_linear_mfma(void* stream, int y_dtype, const void* x, const void* w, void* y, const int* offsets, const int* order,
                        int entries, int experts, int top, int K, int N, int from_tokens, int act, float limit, float alpha);
 int pa_head_linear_mfma(void* stream, const void* x, const void* w, void* y, int tokens, int heads, int K, int N, long xs_t,
@@ -301,7 +305,7 @@ int pa_attn_masked(void* stream, int dtype, const void* q, const void* k_cache, 
                    int table_stride, const int* seq_of_token, const int* positions, void* out, long out_stride, int tokens,
                    int nh, int nkv, int hd, int vd, int page_size, int window, int keep_first, float scale, float softcap,
                    const float* slopes, const float* sink, const void* gate, long gate_stride, float out_scale, const int* cu_q,
-                   const int* context_lens, int nseq, int max_q_len);
+                   const int* context_lens, int nseq, int max_q_len, int nv);
 int pa_attn_masked_mfma_supports(int hd, int vd, int page_size);
 int pa_qkv_prepare(void* stream, int dtype, const void* p, long stride, int q_off, int k_off, int v_off, const float* qw,
                    const float* kw, const int* slots, void* q_out, void* k_cache, void* v_cache, int tokens, int nh, int nkv,
@@ -317,6 +321,24 @@ int pa_gated_delta(void* stream, const float* x, const float* decay, const float
 int pa_rotate_halves_f32(void* stream, int dtype, const void* p, long stride, int q_off, int k_off, int v_off,
                          const float* inv_freq, const int* positions, float* out, int tokens, int heads, int d, int e, int rot,
                          float k_scale);
+
+// ---- parts around a 32-bit stream, in front of and behind attention (stream_parts.hip) ----
+int pa_pair_embed(void* stream, int dtype, const int* ids, const int* positions, const int* seq_of_token, const int* cu_q,
+                  const int* state_slots, int* prev_state, const void* table, const void* pair, float* out, int tokens,
+                  int hidden, int vocab, int buckets, long mul_prev, long mul_cur, float scale);
+int pa_time_conv_add(void* stream, int dtype, const void* h, const float* w, float* state, const int* seq_of_token,
+                     const int* cu_q, const int* state_slots, void* out, int tokens, int nseq, int channels, int taps);
+int pa_stream_add_row(void* stream, float* x, const float* row, int tokens, int hidden);
+int pa_stream_add_branches(void* stream, int dtype, float* x, const void* a, const void* b, long total);
+int pa_qkv_rope_prepare(void* stream, int dtype, const void* p, long stride, int q_off, int k_off, int v_off,
+                        const float* inv_freq, const int* positions, const int* slots, const float* q_scale, void* q_out,
+                        void* k_cache, void* v_cache, int tokens, int nq, int nk, int nv, int hd, int vd, int rot, int pairs,
+                        int page_size);
+int pa_diff_combine(void* stream, int dtype, const void* a, void* out, int tokens, int heads, int vd, float lambda, float eps,
+                    float scale);
+int pa_sigmoid_gate(void* stream, int dtype, const void* o, long o_stride, const void* gate, long gate_stride, void* out,
+                    int rows, int width);
+int pa_cap_logits(void* stream, float* x, long total, float cap);
 
 #ifdef __cplusplus
 }

@@ -41,7 +41,7 @@ __global__ __launch_bounds__(kMaskedWaves* kWave) void attn_masked_kernel(
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ seq_of_token,
     const int* __restrict__ positions, T* __restrict__ out, size_t out_stride, int nh, int nkv, int hd, int vd,
     int page_size, int window, int keep_first, float scale, float softcap, const float* __restrict__ slopes,
-    const float* __restrict__ sink, const T* __restrict__ gate, size_t gate_stride, float out_scale) {
+    const float* __restrict__ sink, const T* __restrict__ gate, size_t gate_stride, float out_scale, int nv) {
   __shared__ float qs[kMaskedWaves][kMaskedMaxDim];
   __shared__ float ps[kMaskedWaves][kWave];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -59,6 +59,7 @@ __global__ __launch_bounds__(kMaskedWaves* kWave) void attn_masked_kernel(
   const int first_window_chunk = lo / kWave > kept_chunks ? lo / kWave : kept_chunks;
   const int last_chunk = hi / kWave;
   const int kvh = active ? h / (nh / nkv) : 0;
+  const int vh = kvh % nv;   // fewer value heads than key heads: key head k goes with value head k mod nv
   const int* table = block_table + (size_t)seq * table_stride;
   const float slope = (slopes && active) ? slopes[h] : 0.f;
 
@@ -99,7 +100,7 @@ __global__ __launch_bounds__(kMaskedWaves* kWave) void attn_masked_kernel(
         if (cj > hi) break;
         if (!(cj >= lo || cj < kept)) continue;
         const int page = table[cj / page_size];
-        const T* vr = v_cache + ((size_t)page * nkv + kvh) * vd * page_size + (cj % page_size);
+        const T* vr = v_cache + ((size_t)page * nv + vh) * vd * page_size + (cj % page_size);
         const float pj = ps[wave][j];
 #pragma unroll
         for (int e = 0; e < kMaskedMaxDim / kWave; ++e) {
@@ -433,8 +434,10 @@ extern "C" int pa_attn_masked(void* stream, int dtype, const void* q, const void
                               void* out, long out_stride, int tokens, int nh, int nkv, int hd, int vd, int page_size,
                               int window, int keep_first, float scale, float softcap, const float* slopes,
                               const float* sink, const void* gate, long gate_stride, float out_scale, const int* cu_q,
-                              const int* context_lens, int nseq, int max_q_len) {
+                              const int* context_lens, int nseq, int max_q_len, int nv) {
   if (tokens == 0) return 0;
+  if (nv <= 0) nv = nkv;
+  PA_REQUIRE(nkv % nv == 0, "attn_masked: %d key heads are not a multiple of %d value heads", nkv, nv);
   PA_REQUIRE(tokens > 0 && nh > 0 && nkv > 0 && page_size > 0 && table_stride > 0,
              "attn_masked: bad sizes tokens=%d nh=%d nkv=%d page=%d table_stride=%d", tokens, nh, nkv, page_size, table_stride);
   PA_REQUIRE(nh % nkv == 0, "attn_masked: %d query heads are not a multiple of %d KV heads", nh, nkv);
@@ -445,7 +448,7 @@ extern "C" int pa_attn_masked(void* stream, int dtype, const void* q, const void
   PA_REQUIRE(out_stride >= (long)nh * vd && (!gate || gate_stride >= nh), "attn_masked: output stride %ld or gate stride %ld "
              "too small for %d heads of %d", out_stride, gate_stride, nh, vd);
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == kBF16 && pa_attn_masked_mfma_supports(hd, vd, page_size) && cu_q && context_lens && nseq > 0 && max_q_len > 0) {
+  if (dtype == kBF16 && nv == nkv && pa_attn_masked_mfma_supports(hd, vd, page_size) && cu_q && context_lens && nseq > 0 && max_q_len > 0) {
     const int group = nh / nkv;
     // two heads a wavefront where the group is even: four leave a head of 128 no registers and measured slower
     const int gt = group % 2 == 0 ? 2 : 1;
@@ -478,12 +481,12 @@ extern "C" int pa_attn_masked(void* stream, int dtype, const void* q, const void
     hipLaunchKernelGGL(attn_masked_kernel<float>, grid, dim3(kMaskedWaves * kWave), 0, st, (const float*)q,
                        (const float*)k_cache, (const float*)v_cache, block_table, table_stride, seq_of_token, positions,
                        (float*)out, (size_t)out_stride, nh, nkv, hd, vd, page_size, window, keep_first, scale, softcap, slopes,
-                       sink, (const float*)gate, (size_t)gate_stride, out_scale);
+                       sink, (const float*)gate, (size_t)gate_stride, out_scale, nv);
   } else if (dtype == kBF16) {
     hipLaunchKernelGGL(attn_masked_kernel<bf16>, grid, dim3(kMaskedWaves * kWave), 0, st, (const bf16*)q,
                        (const bf16*)k_cache, (const bf16*)v_cache, block_table, table_stride, seq_of_token, positions,
                        (bf16*)out, (size_t)out_stride, nh, nkv, hd, vd, page_size, window, keep_first, scale, softcap, slopes,
-                       sink, (const bf16*)gate, (size_t)gate_stride, out_scale);
+                       sink, (const bf16*)gate, (size_t)gate_stride, out_scale, nv);
   } else {
     return pa::fail("attn_masked: unknown element type code %d", dtype);
   }

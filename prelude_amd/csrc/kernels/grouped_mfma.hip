@@ -98,8 +98,10 @@ __device__ __forceinline__ void grouped_tile(const bf16* __restrict__ x, const b
         const int n = nb + 16 * j + 4 * g + i;
         if (n < N) {
           float v = acc[j][mt][i];
-          if (act == 2) {   // a lane's four outputs are two (gate, up) pairs: one output a pair, rows of N / 2
-            if ((i & 1) == 0) y[yo + n / 2] = from_f32<TY>(clamped_gate(v, acc[j][mt][i | 1], limit, alpha));
+          if (act >= 2) {   // a lane's four outputs are two (gate, up) pairs: one output a pair, rows of N / 2
+            if ((i & 1) == 0)
+              y[yo + n / 2] = from_f32<TY>(act == 2 ? clamped_gate(v, acc[j][mt][i | 1], limit, alpha)
+                                                    : gate_activation(v, kActSilu) * acc[j][mt][i | 1]);
             continue;
           }
           if (act == 1) {
@@ -171,7 +173,7 @@ __global__ __launch_bounds__(256) void moe_linear_mfma_kernel(const bf16* __rest
   if (!find_tile(offsets, experts, kGmRows, item % tiles_max, e, p0, p1)) return;
   grouped_tile<TY, NT>(x, w + (size_t)e * N * K, y, K, N, p1 - p0, col_chunk * 64 * NT, act, limit, alpha,
                    [&](int m) { return (long)(from_tokens ? order[p0 + m] / top : p0 + m) * K; },
-                   [&](int m) { return (long)(p0 + m) * (act == 2 ? N / 2 : N); });
+                   [&](int m) { return (long)(p0 + m) * (act >= 2 ? N / 2 : N); });
 }
 
 // The experts' product for many rows: a workgroup owns 128 positions of one expert and 128 outputs.  What limits
@@ -286,7 +288,7 @@ __global__ __launch_bounds__(256) void moe_linear_mfma_big_kernel(const bf16* __
 #pragma unroll
   for (int mt = 0; mt < 8; ++mt) {
     if (mt * 16 + r >= n_rows) continue;
-    TY* yr = y + (size_t)(p0 + mt * 16 + r) * (act == 2 ? N / 2 : N);
+    TY* yr = y + (size_t)(p0 + mt * 16 + r) * (act >= 2 ? N / 2 : N);
 #pragma unroll
     for (int j = 0; j < NT; ++j)
 #pragma unroll
@@ -294,8 +296,10 @@ __global__ __launch_bounds__(256) void moe_linear_mfma_big_kernel(const bf16* __
         const int n = nb + 16 * j + 4 * g + i;
         if (n < N) {
           float v = acc[j][mt][i];
-          if (act == 2) {
-            if ((i & 1) == 0) yr[n / 2] = from_f32<TY>(clamped_gate(v, acc[j][mt][i | 1], limit, alpha));
+          if (act >= 2) {
+            if ((i & 1) == 0)
+              yr[n / 2] = from_f32<TY>(act == 2 ? clamped_gate(v, acc[j][mt][i | 1], limit, alpha)
+                                                : gate_activation(v, kActSilu) * acc[j][mt][i | 1]);
             continue;
           }
           if (act == 1) {
@@ -332,8 +336,9 @@ extern "C" int pa_moe_linear_mfma(void* stream, int y_dtype, const void* x, cons
   if (entries == 0) return 0;
   PA_REQUIRE(entries > 0 && experts > 0 && top > 0 && K > 0 && N > 0 && K % 8 == 0, "moe_linear_mfma: bad sizes entries=%d experts=%d k=%d n=%d",
              entries, experts, K, N);
-  PA_REQUIRE(act == 0 || act == 1 || act == 2, "moe_linear_mfma: unknown activation code %d", act);
-  PA_REQUIRE(act != 2 || (N % 2 == 0 && limit > 0.f), "moe_linear_mfma: gated pairs need an even number of outputs and a clamp > 0");
+  PA_REQUIRE(act >= 0 && act <= 3, "moe_linear_mfma: unknown activation code %d", act);
+  PA_REQUIRE(act < 2 || N % 2 == 0, "moe_linear_mfma: gated pairs need an even number of outputs");
+  PA_REQUIRE(act != 2 || limit > 0.f, "moe_linear_mfma: clamped gated pairs need a clamp > 0");
   const bool few = entries <= 4 * kGmRows;
   const int cols = 128;
   const int col_chunks = (N + cols - 1) / cols;

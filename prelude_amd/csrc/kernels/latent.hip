@@ -32,11 +32,11 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(const T* __restrict__ 
                                                          const int* __restrict__ positions, const int* __restrict__ slots,
                                                          T* __restrict__ cq_out, T* __restrict__ cache,
                                                          T* __restrict__ cache_t, int page_size, int q_rank,
-                                                         int rank, int rot, int rot_dims, float eps) {
+                                                         int rank, int rot, int rot_dims, float eps, size_t in_stride) {
   __shared__ float scratch[16];
   const int t = blockIdx.x;
   const int width = q_rank + rank + rot;
-  const T* row = in + (size_t)t * width;
+  const T* row = in + (size_t)t * in_stride;   // the row may lie inside a wider one
   float sq = 0.f, sc = 0.f;
   for (int i = threadIdx.x; i < q_rank; i += blockDim.x) {
     const float v = to_f32(row[i]);
@@ -257,8 +257,11 @@ using namespace pa;
 
 extern "C" int pa_latent_prep(void* stream, int dtype, const void* in, const float* wq, const float* wc,
                               const float* inv_freq, const int* positions, const int* slots, void* cq_out, void* cache,
-                              void* cache_t, int page_size, int tokens, int q_rank, int rank, int rot, int rot_dims, float eps) {
+                              void* cache_t, int page_size, int tokens, int q_rank, int rank, int rot, int rot_dims, float eps,
+                              long in_stride) {
   if (tokens == 0) return 0;
+  if (in_stride <= 0) in_stride = q_rank + rank + rot;
+  PA_REQUIRE(in_stride >= q_rank + rank + rot, "latent_prep: a row stride of %ld is less than the row", in_stride);
   PA_REQUIRE(tokens > 0 && q_rank > 0 && rank > 0 && rot >= 0, "latent_prep: bad sizes tokens=%d q_rank=%d rank=%d rot=%d",
              tokens, q_rank, rank, rot);
   PA_REQUIRE(rot_dims >= 0 && rot_dims <= rot && rot_dims % 2 == 0, "latent_prep: %d rotated of %d is not an even part", rot_dims, rot);
@@ -267,7 +270,7 @@ extern "C" int pa_latent_prep(void* stream, int dtype, const void* in, const flo
   PA_BY_TYPE(dtype, "latent_prep",
              hipLaunchKernelGGL(latent_prep_kernel<T>, dim3(tokens), dim3(256), 0, (hipStream_t)stream, (const T*)in, wq, wc,
                                 inv_freq, positions, slots, (T*)cq_out, (T*)cache, (T*)cache_t, page_size, q_rank, rank, rot,
-                                rot_dims, eps));
+                                rot_dims, eps, (size_t)in_stride));
   return check_launch("latent_prep");
 }
 

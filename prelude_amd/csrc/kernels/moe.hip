@@ -39,7 +39,7 @@ constexpr int kRouteMax = kRoutePerLane * kWave;
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ correction,
                                                        int* __restrict__ choice, float* __restrict__ weights,
                                                        float* __restrict__ gate_out, int tokens, int experts, int top,
-                                                       float scale, int gate_col) {
+                                                       float scale, int gate_col, const float* __restrict__ bias, int by_logit) {
   const int lane = threadIdx.x % kWave;
   const int t = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
   if (t >= tokens) return;
@@ -49,7 +49,8 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
 #pragma unroll
   for (int j = 0; j < kRoutePerLane; ++j) {
     const int e = lane + j * kWave;
-    s[j] = e < experts ? z[e] : -INFINITY;
+    s[j] = e < experts ? z[e] + (bias ? bias[e] : 0.f) : -INFINITY;
+    c[j] = s[j];   // by_logit: the choice goes by the logit itself
     m = fmaxf(m, s[j]);
   }
   m = wave_max(m);
@@ -64,6 +65,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
 #pragma unroll
   for (int j = 0; j < kRoutePerLane; ++j) {
     const int e = lane + j * kWave;
+    if (by_logit) continue;   // s stays exp(logit - max): over the chosen ones' sum it is the softmax over them alone
     s[j] = s[j] / sum;
     c[j] = e < experts ? s[j] + (correction ? correction[e] : 0.f) : -INFINITY;
   }
@@ -302,14 +304,16 @@ extern "C" int pa_moe_linear(void* stream, int x_dtype, int w_dtype, int y_dtype
 }
 
 extern "C" int pa_moe_route(void* stream, const float* logits, int ld, const float* correction, int* choice, float* weights,
-                            float* gate_out, int tokens, int experts, int top, float scale, int gate_col) {
+                            float* gate_out, int tokens, int experts, int top, float scale, int gate_col, const float* bias,
+                            int by_logit) {
   if (tokens == 0) return 0;
+  PA_REQUIRE(!(by_logit && correction), "moe_route: a choice by the logits takes no correction");
   PA_REQUIRE(tokens > 0 && experts > 0 && top > 0 && top <= experts && ld >= experts, "moe_route: bad sizes tokens=%d experts=%d top=%d ld=%d",
              tokens, experts, top, ld);
   PA_REQUIRE(experts <= kRouteMax, "moe_route: %d experts are more than the %d the kernel takes", experts, kRouteMax);
   PA_REQUIRE(gate_col < ld, "moe_route: gate column %d is outside rows of %d", gate_col, ld);
   hipLaunchKernelGGL(moe_route_kernel, dim3((tokens + 3) / 4), dim3(256), 0, (hipStream_t)stream, logits, ld, correction, choice,
-                     weights, gate_out, tokens, experts, top, scale, gate_col);
+                     weights, gate_out, tokens, experts, top, scale, gate_col, bias, by_logit ? 1 : 0);
   return check_launch("moe_route");
 }
 

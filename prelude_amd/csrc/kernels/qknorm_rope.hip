@@ -28,7 +28,7 @@ __global__ void qknorm_rope_kv_kernel(const T* __restrict__ qkv, const float* __
                                       const int* __restrict__ slots, T* __restrict__ q_out,
                                       T* __restrict__ k_cache, T* __restrict__ v_cache, int tokens, int nh, int nkv,
                                       int hd, int rot, int page_size, float eps, const float* __restrict__ inv_freq,
-                                      int v_from_k) {
+                                      int v_from_k, const float* __restrict__ q_scale) {
   __shared__ float normed[kQkWaves][kMaxHeadDim];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int heads = nh + 2 * nkv;
@@ -102,6 +102,7 @@ __global__ void qknorm_rope_kv_kernel(const T* __restrict__ qkv, const float* __
   const int pos = rot > 0 ? positions[t] : 0;
   const float* c = cos_table ? cos_table + (size_t)pos * half : nullptr;
   const float* s = sin_table ? sin_table + (size_t)pos * half : nullptr;
+  const float mul = (q_scale && h < nh) ? q_scale[h] : 1.0f;   // a number per query head (a temperature), before rounding
 #pragma unroll
   for (int e = 0; e < kMaxHeadDim / kWave; ++e) {
     const int i = lane + e * kWave;
@@ -117,7 +118,7 @@ __global__ void qknorm_rope_kv_kernel(const T* __restrict__ qkv, const float* __
       }
       r = i < half ? x[e] * cj - normed[wave][i + half] * sj : normed[wave][j] * sj + x[e] * cj;
     }
-    dst[i] = from_f32<T>(r);
+    dst[i] = from_f32<T>(r * mul);
   }
 }
 
@@ -308,7 +309,7 @@ static int qknorm_rope_kv_launch(void* stream, int dtype, const void* qkv, const
                                  const float* k_weight, const float* cos_table, const float* sin_table,
                                  const int* positions, const int* slots, void* q_out, void* k_cache,
                                  void* v_cache, int tokens, int nh, int nkv, int hd, int rot, int page_size,
-                                 float eps, const float* inv_freq, int v_from_k) {
+                                 float eps, const float* inv_freq, int v_from_k, const float* q_scale = nullptr) {
   if (tokens == 0) return 0;
   PA_REQUIRE(tokens > 0 && nh > 0 && nkv >= 0 && page_size > 0, "qknorm_rope_kv: bad sizes tokens=%d nh=%d nkv=%d page=%d",
              tokens, nh, nkv, page_size);
@@ -357,11 +358,11 @@ static int qknorm_rope_kv_launch(void* stream, int dtype, const void* qkv, const
   if (dtype == kF32) {
     hipLaunchKernelGGL(qknorm_rope_kv_kernel<float>, dim3(blocks), dim3(kQkWaves * kWave), 0, st, (const float*)qkv,
                        q_weight, k_weight, cos_table, sin_table, positions, slots, (float*)q_out, (float*)k_cache,
-                       (float*)v_cache, tokens, nh, nkv, hd, rot, page_size, eps, inv_freq, v_from_k);
+                       (float*)v_cache, tokens, nh, nkv, hd, rot, page_size, eps, inv_freq, v_from_k, q_scale);
   } else if (dtype == kBF16) {
     hipLaunchKernelGGL(qknorm_rope_kv_kernel<bf16>, dim3(blocks), dim3(kQkWaves * kWave), 0, st, (const bf16*)qkv,
                        q_weight, k_weight, cos_table, sin_table, positions, slots, (bf16*)q_out, (bf16*)k_cache,
-                       (bf16*)v_cache, tokens, nh, nkv, hd, rot, page_size, eps, inv_freq, v_from_k);
+                       (bf16*)v_cache, tokens, nh, nkv, hd, rot, page_size, eps, inv_freq, v_from_k, q_scale);
   } else {
     return pa::fail("qknorm_rope_kv: unknown element type code %d", dtype);
   }
@@ -383,8 +384,8 @@ extern "C" int pa_qknorm_rope_kv(void* stream, int dtype, const void* qkv, const
 extern "C" int pa_qknorm_rope_kv_freq(void* stream, int dtype, const void* qkv, const float* q_weight,
                                       const float* k_weight, const float* inv_freq, const int* positions, const int* slots,
                                       void* q_out, void* k_cache, void* v_cache, int tokens, int nh, int nkv, int hd,
-                                      int rot, int page_size, float eps, int v_from_k) {
+                                      int rot, int page_size, float eps, int v_from_k, const float* q_scale) {
   PA_REQUIRE(rot == 0 || inv_freq, "qknorm_rope_kv: rotary frequencies missing");
   return qknorm_rope_kv_launch(stream, dtype, qkv, q_weight, k_weight, nullptr, nullptr, positions, slots, q_out, k_cache,
-                               v_cache, tokens, nh, nkv, hd, rot, page_size, eps, inv_freq, v_from_k ? 1 : 0);
+                               v_cache, tokens, nh, nkv, hd, rot, page_size, eps, inv_freq, v_from_k ? 1 : 0, q_scale);
 }

@@ -1,5 +1,5 @@
 """Model specifications and the generic decoder built from them.  Importing registers the architectures."""
 from .spec import LayerSpec, ModelSpec, PartSpec, RunSpec
-from . import fazopel, libodra, qwen3, tedalix  # noqa: F401  (registration)
+from . import fazopel, libodra, nivasun, qwen3, tedalix  # noqa: F401  (registration)
 
 __all__ = ["LayerSpec", "ModelSpec", "PartSpec", "RunSpec"]

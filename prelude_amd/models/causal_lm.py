@@ -15,7 +15,7 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from ..parts import Block, Part, TensorReq, build_part
-from ..parts.base import PartError, _REGISTRY
+from ..parts.base import VECTOR, PartError, _REGISTRY
 from .spec import ModelSpec, PartSpec
 
 
@@ -63,6 +63,13 @@ class CausalLM:
         # per member that keeps something, and gets them as a tuple in that order
         self.cache_slots: List[Optional[CacheSlot]] = []
         self.run_cache: List[object] = []   # run index -> None | index into cache_slots | tuple of indices
+        # an embedding that keeps something per request (the token before, say) has a cache slot of its own, owned by no run
+        self.embedding_cache: Optional[int] = None
+        ecs = self.embedding.cache_spec() if hasattr(self.embedding, "cache_spec") else None
+        if ecs is not None:
+            self.embedding_cache = len(self.cache_slots)
+            self.cache_slots.append(CacheSlot(-1, ecs))
+        self.stream_rows: Optional[torch.Tensor] = None
         for i, r in enumerate(spec.order):
             mixer = getattr(self.blocks[r.layer], "mixer", None)
             cs = mixer.cache_spec() if mixer is not None else None
@@ -99,6 +106,9 @@ class CausalLM:
                 if name in out and out[name] != req:
                     raise PartError(f"tensor {name!r} is asked for as {out[name]} and as {req}")
                 out[name] = req
+        if self.spec.stream_rows is not None:
+            name, rows = self.spec.stream_rows
+            out[name] = TensorReq((int(rows), self.spec.hidden_size), VECTOR)
         return out
 
     def load(self, fetch, dtype: torch.dtype, device: torch.device) -> None:
@@ -107,6 +117,9 @@ class CausalLM:
         for part, ps in self._parts:
             tensors = {local: fetch(ps.weights[local], req) for local, req in part.tensors().items()}
             part.load(tensors, dtype, device)
+        if self.spec.stream_rows is not None:
+            name, rows = self.spec.stream_rows
+            self.stream_rows = fetch(name, TensorReq((int(rows), self.spec.hidden_size), VECTOR)).contiguous()
         for p in self.shared.values():
             p.prepare(device)
 
@@ -130,6 +143,7 @@ class CausalLM:
         """Kernel launches of one step, about: every run's block by its parts' own counts, and the embedding, the
         final norm and the head."""
         total = self.embedding.LAUNCHES + self.final_norm.LAUNCHES + self.head.LAUNCHES
+        total += sum(1 for r in self.spec.order if r.stream_row is not None)
         for r in self.spec.order:
             b = self.blocks[r.layer]
             total += b.launches() if hasattr(b, "launches") else 1
@@ -157,15 +171,34 @@ class CausalLM:
         return any(getattr(p, "ATOMIC_PREFILL", False) for p, _ in self._parts)
 
     # ---- forward ------------------------------------------------------------
+    def _add_stream_row(self, hidden, residual, row: int):
+        """Adds row ``row`` of the model's stream rows to the stream, in 32-bit and in place.  The stream is what a block
+        that hands it on left (``hidden`` None, a 32-bit residual), or, in front of the first run, the embedding."""
+        from ..ops import kernels as K
+        if residual is None:
+            hidden = K.as_tensor(hidden)
+            stream = hidden if hidden.dtype == torch.float32 else K.to_f32(hidden)
+            return K.stream_add_row_(stream, self.stream_rows[row]), None
+        if hidden is not None or residual.dtype != torch.float32:
+            raise PartError("a row is added to a 32-bit stream that travels alone between blocks")
+        K.stream_add_row_(residual, self.stream_rows[row])
+        return None, residual
+
     def forward(self, step, caches) -> torch.Tensor:
         """Runs the step's tokens; returns float32 logits [W, vocab] at ``step.want_rows``.
 
         ``caches[i]`` is the view of cache slot i (``engine.caches``).
         """
-        hidden = self.embedding.forward(step.token_ids)
+        if getattr(self.embedding, "NEEDS_STEP", False):
+            hidden = self.embedding.forward(step.token_ids, step=step,
+                                            cache=None if self.embedding_cache is None else caches[self.embedding_cache])
+        else:
+            hidden = self.embedding.forward(step.token_ids)
         residual = None
         step.compute_dtype = self.dtype
         for i, r in enumerate(self.spec.order):
+            if r.stream_row is not None:
+                hidden, residual = self._add_stream_row(hidden, residual, r.stream_row)
             ci = self.run_cache[i]
             cache = None if ci is None else (tuple(caches[c] for c in ci) if isinstance(ci, tuple) else caches[ci])
             hidden, residual = self.blocks[r.layer].forward(hidden, residual, step, cache,

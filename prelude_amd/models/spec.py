@@ -32,9 +32,12 @@ class RunSpec:
     ``layer`` may appear in several runs (the same weights applied again).
     Each run has a cache of its own unless ``reads_cache_of`` names an earlier
     run (by its index in ``order``) whose cache it reads without writing.
+    ``stream_row``: row of the model's ``stream_rows`` tensor that is added to the stream right in front of this run
+    (a learned vector per pass of a stretch of layers that runs several times, say); None: nothing.
     """
     layer: int
     reads_cache_of: Optional[int] = None
+    stream_row: Optional[int] = None
 
 
 @dataclasses.dataclass
@@ -53,6 +56,8 @@ class ModelSpec:
     # checkpoint names (shell patterns) that files of this architecture may hold and the model does not read:
     # they are passed over; any other tensor nothing asks for is an error
     ignored_tensors: Tuple[str, ...] = ()
+    # (checkpoint name, rows) of a 32-bit tensor [rows, hidden] whose rows runs may add to the stream (``RunSpec.stream_row``)
+    stream_rows: Optional[Tuple[str, int]] = None
 
     def validate(self) -> None:
         if not self.order:
@@ -60,6 +65,9 @@ class ModelSpec:
         for i, r in enumerate(self.order):
             if not 0 <= r.layer < len(self.layers):
                 raise ValueError(f"model spec: run {i} names layer {r.layer}, there are {len(self.layers)}")
+            if r.stream_row is not None and (self.stream_rows is None or not 0 <= r.stream_row < self.stream_rows[1]):
+                raise ValueError(f"model spec: run {i} adds row {r.stream_row} of a tensor of "
+                                 f"{self.stream_rows[1] if self.stream_rows else 0} rows")
             if r.reads_cache_of is not None:
                 if not 0 <= r.reads_cache_of < i:
                     raise ValueError(f"model spec: run {i} reads the cache of run {r.reads_cache_of}, "

@@ -211,7 +211,8 @@ def qknorm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight
                    cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
                    slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
                    num_heads: int, num_kv_heads: int, head_dim: int, rotary_dim: int, eps: float,
-                   inv_freq: Optional[torch.Tensor] = None, values_from_keys: bool = False) -> torch.Tensor:
+                   inv_freq: Optional[torch.Tensor] = None, values_from_keys: bool = False,
+                   q_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Per-head RMSNorm of Q and K, rotation by position, K and V into the paged cache.
 
     qkv [T, (nh + 2 nkv) * hd]; returns q [T, nh, hd].  With ``slots`` None
@@ -219,9 +220,13 @@ def qknorm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight
     Q-only input).  K cache [pages, nkv, page_size, hd], V cache [pages, nkv, hd, page_size].
     ``inv_freq`` (float32 [rotary_dim / 2]) in place of the tables: the kernel takes the angle
     position * inv_freq[j] and its cosine and sine itself.  ``values_from_keys``: qkv is [T, (nh + nkv) * hd]
-    and a head's cached value is its key as projected, before norm and rotation.
+    and a head's cached value is its key as projected, before norm and rotation.  ``q_scale`` (float32 [nh]): every
+    query head times its number, in 32-bit before it is rounded (a temperature per head).
     """
-    _dev(qkv, q_weight, k_weight, cos, sin, positions, slots, k_cache, v_cache, inv_freq)
+    _dev(qkv, q_weight, k_weight, cos, sin, positions, slots, k_cache, v_cache, inv_freq, q_scale)
+    _f32(q_scale, "query scales")
+    if q_scale is not None and tuple(q_scale.shape) != (num_heads,):
+        raise NativeError(f"qknorm_rope_kv: query scales {tuple(q_scale.shape)} for {num_heads} heads")
     _i32(positions, "positions")
     _f32(q_weight, "q_norm weight")
     _f32(k_weight, "k_norm weight")
@@ -237,7 +242,9 @@ def qknorm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight
     for w, nm in ((q_weight, "q_norm"), (k_weight, "k_norm")):
         if w is not None and w.shape != (head_dim,):
             raise NativeError(f"qknorm_rope_kv: {nm} weight {tuple(w.shape)} is not [{head_dim}]")
-    by_freq = inv_freq is not None or values_from_keys
+    by_freq = inv_freq is not None or values_from_keys or q_scale is not None
+    if q_scale is not None and (cos is not None or sin is not None):
+        raise NativeError("qknorm_rope_kv: a scale per query head goes with rotation from the frequencies, not from tables")
     if rotary_dim and inv_freq is not None:
         if cos is not None or sin is not None or tuple(inv_freq.shape) != (rotary_dim // 2,):
             raise NativeError(f"qknorm_rope_kv: frequencies must be [{rotary_dim // 2}] and come without tables")
@@ -258,7 +265,7 @@ def qknorm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight
         check(kernels().pa_qknorm_rope_kv_freq(_stream(), _code(qkv), _ptr(qkv), _ptr(q_weight), _ptr(k_weight), _ptr(inv_freq),
                                                _ptr(positions), _ptr(slots), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), t,
                                                num_heads, num_kv_heads, head_dim, rotary_dim, page_size, float(eps),
-                                               1 if values_from_keys else 0))
+                                               1 if values_from_keys else 0, _ptr(q_scale)))
         return q_out
     check(kernels().pa_qknorm_rope_kv(_stream(), _code(qkv), _ptr(qkv), _ptr(q_weight), _ptr(k_weight), _ptr(cos),
                                       _ptr(sin), _ptr(positions), _ptr(slots), _ptr(q_out), _ptr(k_cache),
@@ -1239,13 +1246,16 @@ def latent_prep(down: torch.Tensor, q_weight: torch.Tensor, c_weight: torch.Tens
     """The merged down projection [T, q_rank + rank + rot]: returns the normed query latent [T, q_rank]; writes the
     normed latent and the rotated shared key part of every token into ``cache`` [pages, page, rank + rot] at ``slots``,
     and the latent once more into ``cache_t`` [pages, rank, page] where the cache keeps that copy."""
-    _dev(down, q_weight, c_weight, inv_freq, positions, slots, cache, cache_t)
+    _dev(q_weight, c_weight, inv_freq, positions, slots, cache, cache_t)   # ``down`` may be rows of a wider tensor
+    if not down.is_cuda:
+        raise NativeError("latent_prep: the projection is not on the device")
     _f32(q_weight, "query latent norm weight")
     _f32(c_weight, "latent norm weight")
     _f32(inv_freq, "rotary frequencies")
     _i32(positions, "positions")
     t = down.shape[0]
-    if down.dim() != 2 or down.shape[1] != q_rank + rank + rot or q_weight.shape != (q_rank,) or c_weight.shape != (rank,):
+    if down.dim() != 2 or down.shape[1] != q_rank + rank + rot or down.stride(1) != 1 or q_weight.shape != (q_rank,) or \
+            c_weight.shape != (rank,):
         raise NativeError(f"latent_prep: input {tuple(down.shape)} for parts {q_rank} + {rank} + {rot}")
     if positions.shape != (t,) or (rot_dims and (inv_freq is None or inv_freq.shape != (rot_dims // 2,))):
         raise NativeError("latent_prep: positions or rotary frequencies do not match")
@@ -1257,10 +1267,10 @@ def latent_prep(down: torch.Tensor, q_weight: torch.Tensor, c_weight: torch.Tens
             raise NativeError(f"latent_prep: the transposed copy must be [pages, {rank}, page] of {cache.dtype}")
     cq = torch.empty((t, q_rank), dtype=down.dtype, device=down.device)
     caching = slots is not None
-    check(kernels().pa_latent_prep(_stream(), _code(down), _ptr(down), _ptr(q_weight), _ptr(c_weight), _ptr(inv_freq),
+    check(kernels().pa_latent_prep(_stream(), _code(down), down.data_ptr(), _ptr(q_weight), _ptr(c_weight), _ptr(inv_freq),
                                    _ptr(positions), _ptr(slots), _ptr(cq), _ptr(cache) if caching else None,
                                    _ptr(cache_t) if caching else None, cache.shape[1] if caching else 0, t,
-                                   q_rank, rank, rot, rot_dims, float(eps)))
+                                   q_rank, rank, rot, rot_dims, float(eps), down.stride(0)))
     return cq
 
 
@@ -1390,12 +1400,19 @@ def linear_narrow_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
 
 
 def moe_route(logits: torch.Tensor, experts: int, top: int, scale: float, correction: Optional[torch.Tensor] = None,
-              gate_col: int = -1):
+              gate_col: int = -1, bias: Optional[torch.Tensor] = None, by_logit: bool = False):
     """A router's choices: logits float32 [T, >= experts]; s = softmax over the first ``experts`` columns; the ``top``
     experts with the largest s + correction are chosen and weighted s / (sum of the chosen s + 1e-20) * scale.
     Returns (choice int32 [T * top], weights float32 [T * top], gate float32 [T] or None): the gate is the sigmoid of
-    column ``gate_col`` of the same rows, for a shared expert."""
-    _dev(logits, correction)
+    column ``gate_col`` of the same rows, for a shared expert.  ``bias`` (float32 [experts]) is added to the logits
+    first.  ``by_logit``: the choice goes by the logits themselves (no correction) and the weights are the softmax over
+    the chosen logits alone, times scale."""
+    _dev(logits, correction, bias)
+    _f32(bias, "router bias")
+    if bias is not None and tuple(bias.shape) != (experts,):
+        raise NativeError(f"moe_route: bias {tuple(bias.shape)} for {experts} experts")
+    if by_logit and correction is not None:
+        raise NativeError("moe_route: a choice by the logits takes no correction")
     _f32(logits, "router logits")
     _f32(correction, "router correction")
     if logits.dim() != 2 or logits.shape[1] < experts or (correction is not None and tuple(correction.shape) != (experts,)):
@@ -1405,7 +1422,8 @@ def moe_route(logits: torch.Tensor, experts: int, top: int, scale: float, correc
     weights = torch.empty(t * top, dtype=torch.float32, device=logits.device)
     gate = torch.empty(t, dtype=torch.float32, device=logits.device) if gate_col >= 0 else None
     check(kernels().pa_moe_route(_stream(), _ptr(logits), logits.shape[1], _ptr(correction), _ptr(choice), _ptr(weights),
-                                 _ptr(gate), t, int(experts), int(top), float(scale), int(gate_col)))
+                                 _ptr(gate), t, int(experts), int(top), float(scale), int(gate_col), _ptr(bias),
+                                 1 if by_logit else 0))
     return choice, weights, gate
 
 
@@ -1421,33 +1439,38 @@ def moe_order(choice: torch.Tensor, experts: int, top: int) -> ExpertOrder:
 
 
 def moe_linear(x: torch.Tensor, w: GroupedWeight, eo: ExpertOrder, from_tokens: bool, relu_squared_epilogue: bool = False,
-               out_dtype: Optional[torch.dtype] = None, clamped_gate_epilogue: Optional[tuple] = None) -> torch.Tensor:
+               out_dtype: Optional[torch.dtype] = None, clamped_gate_epilogue: Optional[tuple] = None,
+               silu_gate_epilogue: bool = False) -> torch.Tensor:
     """y[p] = act(W[expert of p] x[row of p]) over the ordered positions p; ``w`` [experts, n, k];
     ``from_tokens``: x holds a row per token (position p reads its token's), else a row per position.
     ``clamped_gate_epilogue`` = (limit, alpha): the weights' rows alternate gate_j, up_j and the result is the
     clamped gated pair of ``clamped_gate``, [entries, n / 2] (in the matrix-core product's epilogue; a kernel of
-    its own behind the other product)."""
+    its own behind the other product).  ``silu_gate_epilogue``: the same rows, the plain gated pair
+    silu(gate_j) * up_j."""
     wt = w.nk if w.nk is not None else w.kn
     _dev(x, wt)
     k, n = w.k, w.n
     rows = eo.entries // eo.top if from_tokens else eo.entries
     if x.dim() != 2 or tuple(x.shape) != (rows, k) or w.groups != eo.experts or x.dtype != w.dtype:
         raise NativeError(f"moe_linear: x {tuple(x.shape)} {x.dtype} / w [{w.groups}, {n}, {k}] {w.dtype} for {eo.entries} entries")
-    if clamped_gate_epilogue is not None and (relu_squared_epilogue or n % 2):
+    gated = clamped_gate_epilogue is not None or silu_gate_epilogue
+    if gated and (relu_squared_epilogue or n % 2 or (clamped_gate_epilogue is not None and silu_gate_epilogue)):
         raise NativeError(f"moe_linear: gated pairs over {n} outputs, or two activations at once")
     out_dtype = out_dtype or x.dtype
-    fused = clamped_gate_epilogue is not None and w.nk is not None
+    fused = gated and w.nk is not None
     y = torch.empty((eo.entries, n // 2 if fused else n), dtype=out_dtype, device=x.device)
-    act = 2 if fused else (1 if relu_squared_epilogue else 0)
+    act = (3 if silu_gate_epilogue else 2) if fused else (1 if relu_squared_epilogue else 0)
     args = (_ptr(x), _ptr(wt), _ptr(y), _ptr(eo.offsets), _ptr(eo.order), eo.entries, eo.experts, eo.top, k, n,
             1 if from_tokens else 0, act)
     if w.nk is not None:
-        limit, alpha = clamped_gate_epilogue if fused else (0.0, 0.0)
+        limit, alpha = clamped_gate_epilogue if (fused and clamped_gate_epilogue is not None) else (0.0, 0.0)
         check(kernels().pa_moe_linear_mfma(_stream(), _CODES[out_dtype], *args, float(limit), float(alpha)))
         return y
     check(kernels().pa_moe_linear(_stream(), _code(x), _code(wt), _CODES[out_dtype], *args))
     if clamped_gate_epilogue is not None:
         return clamped_gate(y, *clamped_gate_epilogue)
+    if silu_gate_epilogue:
+        return silu_mul(y)
     return y
 
 
@@ -1696,8 +1719,8 @@ def attention_masked(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
         raise NativeError(f"attention_masked: q {tuple(q.shape)} / caches")
     t, nh, hd = q.shape
     pages, nkv, page, khd = k_cache.shape
-    vd = v_cache.shape[2]
-    if khd != hd or tuple(v_cache.shape) != (pages, nkv, vd, page) or k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
+    nv, vd = v_cache.shape[1], v_cache.shape[2]   # fewer value heads than key heads: key head k goes with value head k mod nv
+    if khd != hd or tuple(v_cache.shape) != (pages, nv, vd, page) or nkv % nv or k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
         raise NativeError(f"attention_masked: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} for q {tuple(q.shape)} {q.dtype}")
     for name, v in (("slopes", slopes), ("sink", sink)):
         if v is not None:
@@ -1717,7 +1740,7 @@ def attention_masked(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                                        float(softcap), _ptr(slopes), _ptr(sink), gate.data_ptr() if gate is not None else None,
                                        gate.stride(0) if gate is not None else 0, float(out_scale), _ptr(getattr(step, "cu_q", None)),
                                        _ptr(getattr(step, "context_lens", None)), int(getattr(step, "num_seqs", 0)),
-                                       int(getattr(step, "max_q_len", 0) or getattr(step, "max_prefill_q", 0) or 1)))
+                                       int(getattr(step, "max_q_len", 0) or getattr(step, "max_prefill_q", 0) or 1), nv))
     return out
 
 
@@ -1790,3 +1813,134 @@ def rotate_halves_f32(p: torch.Tensor, q_off: int, k_off: int, v_off: int, inv_f
         check(kernels().pa_rotate_halves_f32(_stream(), _code(p), p.data_ptr(), p.stride(0), int(q_off), int(k_off), int(v_off),
                                              _ptr(inv_freq), _ptr(positions), _ptr(out), t, heads, d, e, int(rot), float(k_scale)))
     return out
+
+
+# ---------------------------------------------------------------------------
+# Parts around a 32-bit stream, in front of and behind attention
+def pair_embed(ids: torch.Tensor, step, prev_state: torch.Tensor, table: torch.Tensor, pair: torch.Tensor, buckets: int,
+               mul_prev: int, mul_cur: int, scale: float) -> torch.Tensor:
+    """out[t] = table[ids[t]] * scale + pair[(prev * mul_prev + ids[t] * mul_cur) mod buckets] in 32-bit, [T, H]; a
+    sequence's first token (position 0) reads row ``buckets`` of ``pair``.  The token before a portion's first comes
+    from ``prev_state`` (int32 [slots, 1], the step's ``state_slots``), which then takes the portion's last token."""
+    _dev(ids, table, pair, prev_state, step.positions, step.seq_of_token, step.cu_q, step.state_slots)
+    _i32(ids, "ids")
+    _i32(prev_state, "previous tokens")
+    t, h = ids.shape[0], table.shape[1]
+    if ids.dim() != 1 or table.dim() != 2 or tuple(pair.shape) != (buckets + 1, h) or pair.dtype != table.dtype:
+        raise NativeError(f"pair_embed: ids {tuple(ids.shape)} / table {tuple(table.shape)} / pair {tuple(pair.shape)} for {buckets} buckets")
+    out = torch.empty((t, h), dtype=torch.float32, device=table.device)
+    check(kernels().pa_pair_embed(_stream(), _code(table), _ptr(ids), _ptr(step.positions), _ptr(step.seq_of_token), _ptr(step.cu_q),
+                                  _ptr(step.state_slots), _ptr(prev_state), _ptr(table), _ptr(pair), _ptr(out), t, h, table.shape[0],
+                                  int(buckets), int(mul_prev), int(mul_cur), float(scale)))
+    return out
+
+
+def time_conv_add(h: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Tensor], step) -> torch.Tensor:
+    """h + conv(h) with conv(h)_t = sum_j w[:, j] h_(t - taps + 1 + j) over time within each sequence, zeros before its
+    start.  h [T, C]; ``weight`` float32 [C, taps]; ``state`` float32 [slots, taps - 1, C]: a request's last taps - 1
+    inputs, read for the places before the portion and moved on afterwards."""
+    _dev(h, weight, state, step.seq_of_token, step.cu_q, step.state_slots)
+    _f32(weight, "convolution weight")
+    _f32(state, "carried inputs")
+    t, c = h.shape
+    taps = weight.shape[1]
+    if weight.dim() != 2 or weight.shape[0] != c or not h.is_contiguous() or \
+            (taps > 1 and (state is None or tuple(state.shape[1:]) != (taps - 1, c))):
+        raise NativeError(f"time_conv_add: h {tuple(h.shape)} / weight {tuple(weight.shape)} / state "
+                          f"{None if state is None else tuple(state.shape)}")
+    out = torch.empty_like(h)
+    check(kernels().pa_time_conv_add(_stream(), _code(h), _ptr(h), _ptr(weight), _ptr(state), _ptr(step.seq_of_token), _ptr(step.cu_q),
+                                     _ptr(step.state_slots), _ptr(out), t, int(step.num_seqs), c, taps))
+    return out
+
+
+def stream_add_row_(x: torch.Tensor, row: torch.Tensor) -> torch.Tensor:
+    """x[t] += row for every row of a 32-bit stream x [T, H], in place."""
+    _dev(x, row)
+    _f32(x, "stream")
+    _f32(row, "row")
+    if x.dim() != 2 or tuple(row.shape) != (x.shape[1],) or not x.is_contiguous() or not row.is_contiguous():
+        raise NativeError(f"stream_add_row: x {tuple(x.shape)} / row {tuple(row.shape)}")
+    check(kernels().pa_stream_add_row(_stream(), _ptr(x), _ptr(row), x.shape[0], x.shape[1]))
+    return x
+
+
+def stream_add_branches_(x: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x += a + b (the branches' sum first, in 32-bit) for a 32-bit stream x [T, H], in place."""
+    _dev(x, a, b)
+    _f32(x, "stream")
+    if a.shape != x.shape or not a.is_contiguous() or not x.is_contiguous() or \
+            (b is not None and (b.shape != x.shape or b.dtype != a.dtype or not b.is_contiguous())):
+        raise NativeError(f"stream_add_branches: x {tuple(x.shape)} / a {tuple(a.shape)} / b {None if b is None else tuple(b.shape)}")
+    check(kernels().pa_stream_add_branches(_stream(), _code(a), _ptr(x), _ptr(a), _ptr(b), x.numel()))
+    return x
+
+
+def qkv_rope_prepare(p: torch.Tensor, q_off: int, k_off: int, v_off: int, inv_freq: Optional[torch.Tensor], positions: torch.Tensor,
+                     slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], nq: int,
+                     nk: int, nv: int, hd: int, vd: int, rot: int, pairs: bool, q_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """From the merged projection ``p`` [T, width]: the queries [T, nq, hd]; ``nk`` key heads of ``hd`` into K
+    [pages, nk, page, hd] and ``nv`` value heads of ``vd`` into V [pages, nv, vd, page] at ``slots`` (None: queries
+    only).  The first ``rot`` dimensions of every query and key head are turned by position * inv_freq[i], dimension i
+    with i + rot / 2, or with ``pairs`` 2i with 2i + 1; ``q_scale`` [nq]: a number per query head."""
+    _dev(p, inv_freq, positions, slots, k_cache, v_cache, q_scale)
+    _f32(inv_freq, "rotary frequencies")
+    _f32(q_scale, "query scales")
+    _i32(positions, "positions")
+    if p.dim() != 2 or p.stride(1) != 1:
+        raise NativeError(f"qkv_rope_prepare: projection {tuple(p.shape)} with strides {p.stride()}")
+    t = p.shape[0]
+    if rot and (inv_freq is None or tuple(inv_freq.shape) != (rot // 2,)):
+        raise NativeError(f"qkv_rope_prepare: frequencies must be [{rot // 2}]")
+    if q_scale is not None and tuple(q_scale.shape) != (nq,):
+        raise NativeError(f"qkv_rope_prepare: query scales {tuple(q_scale.shape)} for {nq} heads")
+    page = 0
+    if slots is not None:
+        _i32(slots, "slots")
+        if slots.shape != (t,) or k_cache is None or v_cache is None or k_cache.dtype != p.dtype or v_cache.dtype != p.dtype or \
+                tuple(k_cache.shape[1:]) != (nk, k_cache.shape[2], hd) or tuple(v_cache.shape) != (k_cache.shape[0], nv, vd, k_cache.shape[2]):
+            raise NativeError(f"qkv_rope_prepare: caches {None if k_cache is None else tuple(k_cache.shape)} / "
+                              f"{None if v_cache is None else tuple(v_cache.shape)} for {nk} key heads of {hd} and {nv} value heads of {vd}")
+        page = k_cache.shape[2]
+    q = torch.empty((t, nq, hd), dtype=p.dtype, device=p.device)
+    if t:
+        caching = slots is not None
+        check(kernels().pa_qkv_rope_prepare(_stream(), _code(p), p.data_ptr(), p.stride(0), int(q_off), int(k_off), int(v_off),
+                                            _ptr(inv_freq), _ptr(positions), _ptr(slots), _ptr(q_scale), _ptr(q),
+                                            _ptr(k_cache) if caching else None, _ptr(v_cache) if caching else None, t, nq, nk, nv,
+                                            hd, vd, int(rot), 1 if pairs else 0, page))
+    return q
+
+
+def diff_combine(a: torch.Tensor, heads: int, lam: float, eps: float, scale: float) -> torch.Tensor:
+    """a [T, 2 * heads * vd] (the first maps' outputs of all heads, then the second maps') -> [T, heads * vd]:
+    u = a1 - lam * a2 per head, over its own sqrt(mean(u^2) + eps), times ``scale``."""
+    _dev(a)
+    if a.dim() != 2 or a.shape[1] % (2 * heads) or not a.is_contiguous():
+        raise NativeError(f"diff_combine: a {tuple(a.shape)} for {heads} heads")
+    vd = a.shape[1] // (2 * heads)
+    out = torch.empty((a.shape[0], heads * vd), dtype=a.dtype, device=a.device)
+    check(kernels().pa_diff_combine(_stream(), _code(a), _ptr(a), _ptr(out), a.shape[0], heads, vd, float(lam), float(eps), float(scale)))
+    return out
+
+
+def sigmoid_gate(o: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """o * sigmoid(gate), element by element; both [T, N], rows may lie inside wider tensors."""
+    if not (o.is_cuda and gate.is_cuda):
+        raise NativeError("sigmoid_gate: an operand is not on the device")
+    if o.dim() != 2 or o.shape != gate.shape or o.dtype != gate.dtype or o.stride(1) != 1 or gate.stride(1) != 1:
+        raise NativeError(f"sigmoid_gate: o {tuple(o.shape)} {o.dtype} / gate {tuple(gate.shape)} {gate.dtype}")
+    out = torch.empty(o.shape, dtype=o.dtype, device=o.device)
+    check(kernels().pa_sigmoid_gate(_stream(), _code(o), o.data_ptr(), o.stride(0), gate.data_ptr(), gate.stride(0), _ptr(out),
+                                    o.shape[0], o.shape[1]))
+    return out
+
+
+def cap_logits_(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """x <- cap * tanh(x / cap) for 32-bit logits, in place."""
+    _dev(x)
+    _f32(x, "logits")
+    if not x.is_contiguous():
+        raise NativeError("cap_logits: the logits are not contiguous")
+    check(kernels().pa_cap_logits(_stream(), _ptr(x), x.numel(), float(cap)))
+    return x

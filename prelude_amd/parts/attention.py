@@ -29,7 +29,7 @@ class GQAAttention(Mixer):
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, norm_eps: float = 1e-6,
                  qk_norm: bool = True, bias: bool = False, window: int = 0, position: Optional[str] = None,
                  rotary_dim: Optional[int] = None, scale: Optional[float] = None, score_cap: float = 0.0,
-                 values_from_keys: bool = False, sink: Optional[str] = None):
+                 values_from_keys: bool = False, sink: Optional[str] = None, head_scale: bool = False):
         if num_heads % num_kv_heads:
             raise PartError(f"gqa_attention: {num_heads} heads are not a multiple of {num_kv_heads} KV heads")
         # what the kernels take: the matrix-core attention has head sizes of its own (others go to the generic
@@ -54,10 +54,13 @@ class GQAAttention(Mixer):
         if sink not in (None, "zero", "learned"):
             raise PartError(f"gqa_attention: sink {sink!r} is not one of None, 'zero', 'learned'")
         self.sink = sink
+        # a learned number per query head that its scores are multiplied by (a temperature), tensor ``head_scales``
+        # [heads]: the rotated queries take it in 32-bit before they are rounded
+        self.head_scale = bool(head_scale)
         if self.values_from_keys and self.bias:
             raise PartError("gqa_attention: values that are the keys come without biases")
         self.rope = None
-        self.w_qkv = self.b_qkv = self.w_o = self.b_o = self.q_norm = self.k_norm = self.sinks = None
+        self.w_qkv = self.b_qkv = self.w_o = self.b_o = self.q_norm = self.k_norm = self.sinks = self.head_scales = None
 
     def cache_spec(self):
         return KVCacheSpec(self.num_kv_heads, self.head_dim, self.window)
@@ -67,9 +70,9 @@ class GQAAttention(Mixer):
             if self.position not in shared:
                 raise PartError(f"gqa_attention: the model has no position encoding named {self.position!r}")
             self.rope = shared[self.position]
-            if self.values_from_keys and not hasattr(self.rope, "inv_freq"):
-                raise PartError("gqa_attention: values that are the keys take their rotation from frequencies "
-                                "(a position encoding that offers `inv_freq`), not from tables")
+            if (self.values_from_keys or self.head_scale) and not hasattr(self.rope, "inv_freq"):
+                raise PartError("gqa_attention: values that are the keys, and a scale per head, take their rotation from "
+                                "frequencies (a position encoding that offers `inv_freq`), not from tables")
             if getattr(self.rope, "rotary_dim", None) != self.rotary_dim:
                 raise PartError(f"gqa_attention: position encoding {self.position!r} has width "
                                 f"{getattr(self.rope, 'rotary_dim', None)}, the mixer rotates {self.rotary_dim}")
@@ -82,6 +85,8 @@ class GQAAttention(Mixer):
             del t["v_proj.weight"]
         if self.sink == "learned":
             t["sinks"] = TensorReq((nh,), VECTOR)
+        if self.head_scale:
+            t["head_scales"] = TensorReq((nh,), NORM)
         if self.bias:
             t.update({"q_proj.bias": TensorReq((nh * hd,), VECTOR), "k_proj.bias": TensorReq((nkv * hd,), VECTOR),
                       "v_proj.bias": TensorReq((nkv * hd,), VECTOR), "o_proj.bias": TensorReq((h,), VECTOR)})
@@ -99,6 +104,8 @@ class GQAAttention(Mixer):
         elif self.sink == "zero":
             self.sinks = torch.zeros(self.num_heads, dtype=torch.float32, device=device)
         self.w_o = K.prepare_weight(tensors["o_proj.weight"])
+        if self.head_scale:
+            self.head_scales = tensors["head_scales"]
         if self.bias:
             self.b_qkv = torch.cat([tensors["q_proj.bias"], tensors["k_proj.bias"], tensors["v_proj.bias"]]).contiguous()
             self.b_o = tensors["o_proj.bias"]
@@ -112,6 +119,7 @@ class GQAAttention(Mixer):
         rotation that every workgroup of the attention kernel then does for itself."""
         return (x.dtype == torch.bfloat16 and self.rope is not None and step.decode_seqs is not None
                 and getattr(self.rope, "cos", None) is not None and not self.values_from_keys and self.sinks is None
+                and self.head_scales is None
                 and step.n_prefill == 0 and step.n_decode == step.num_seqs <= self.FUSED_DECODE_MAX_SEQS
                 and K.attention_decode_fused_supported(self.num_heads, self.num_kv_heads, self.head_dim,
                                                        self.rotary_dim, cache.k.shape[2]))
@@ -124,6 +132,8 @@ class GQAAttention(Mixer):
         sin = getattr(self.rope, "sin", None) if self.rope is not None else None
         freq = getattr(self.rope, "inv_freq", None) if self.rope is not None and cos is None else None
         how = dict(inv_freq=freq, values_from_keys=self.values_from_keys) if (freq is not None or self.values_from_keys) else {}
+        if self.head_scales is not None:
+            how["q_scale"] = self.head_scales
         if write_cache and self._fused_decode(x, step, cache):
             # a step of single tokens: the norm, the rotation and the cache write happen inside the attention kernel
             qkv = K.linear(x, self.w_qkv, self.b_qkv)
@@ -139,8 +149,11 @@ class GQAAttention(Mixer):
         else:  # reads keys and values another layer wrote: only the queries are projected
             bq = self.b_qkv[: nh * hd] if self.b_qkv is not None else None
             qx = K.linear(x, self.w_qkv.first_rows(nh * hd), bq)
+            only_q = {"inv_freq": freq} if freq is not None else {}
+            if self.head_scales is not None:
+                only_q["q_scale"] = self.head_scales
             q = K.qknorm_rope_kv(qx, self.q_norm, None, cos, sin, step.positions, None, None, None, nh, 0, hd,
-                                 self.rotary_dim, self.norm_eps, **({"inv_freq": freq} if freq is not None else {}))
+                                 self.rotary_dim, self.norm_eps, **only_q)
         o = K.attention(q, cache.k, cache.v, g, step, self.window, self.scale, self.score_cap, sink=self.sinks)
         return K.linear(o.view(o.shape[0], nh * hd), self.w_o, self.b_o, slices_ok=True)
 
@@ -270,3 +283,98 @@ class WindowedAttention(Mixer):
     def forward(self, x, step, cache, write_cache=True):
         p = K.linear(x, self.w_in)
         return K.linear(self.mix(x, p, 0, step, cache, write_cache), self.w_o, slices_ok=True)
+
+
+@dataclasses.dataclass(frozen=True)
+class SharedValueKVCacheSpec(KVCacheSpec):
+    """Keys and values in pages where several key heads read one value head: ``num_kv_heads`` key heads of ``head_dim``
+    and ``num_value_heads`` value heads of ``value_dim`` (key head k goes with value head k mod ``num_value_heads``).
+    K ``[pages, key heads, page, head_dim]``, V ``[pages, value heads, value width, page]``."""
+    num_value_heads: int = 0
+
+    def bytes_per_token(self, element_size: int) -> int:
+        return (self.num_kv_heads * self.head_dim + self.num_value_heads * self.v_dim) * element_size
+
+    def allocate(self, pages, page_size, dtype, device, group):
+        from .base import KVLayerCache
+        return KVLayerCache(torch.zeros((pages, self.num_kv_heads, page_size, self.head_dim), dtype=dtype, device=device),
+                            torch.zeros((pages, self.num_value_heads, self.v_dim, page_size), dtype=dtype, device=device), group)
+
+
+@register_part("mixer", "differential_attention")
+class DifferentialAttention(Mixer):
+    """Two attention maps a head over the same values, one taken off the other.  The query projection has
+    heads * 2 * head_dim rows and the key projection kv_heads * 2 * head_dim, laid out head by head as [map 1 | map 2];
+    the value projection kv_heads * value_dim.  The first ``rotary_dim`` dimensions of every map of every query and key
+    head are turned by position, dimension 2i with 2i + 1.  Each map is a softmax attention of its own under the window
+    (score = q.k * scale); with a1, a2 their outputs and lambda = exp(lq1.lk1) - exp(lq2.lk2) + ``diff`` (one number a
+    layer, from four learned vectors of head_dim), a head's output is u = a1 - lambda a2 over its own
+    sqrt(mean(u^2) + eps), times 1 - ``diff``.
+
+    The maps run as 2 * heads query heads over 2 * kv_heads key heads (the projections' rows put map-major when they are
+    loaded) whose value head is the key head modulo kv_heads: the values are cached once."""
+    LAUNCHES = 5   # merged projection, rotation + cache write, attention, the maps' difference and norm, output projection
+    GRAPH_SAFE_PORTIONS = True
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, scale: float,
+                 diff: float, norm_eps: float, window: int = 0, position: Optional[str] = None, rotary_dim: int = 0):
+        if num_heads % num_kv_heads:
+            raise PartError(f"differential_attention: {num_heads} heads are not a multiple of {num_kv_heads} KV heads")
+        if not (1 <= head_dim <= 256 and 1 <= value_dim <= 256):
+            raise PartError(f"differential_attention: key width {head_dim} or value width {value_dim} is outside 1..256")
+        self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.head_dim, self.value_dim, self.scale, self.diff = int(head_dim), int(value_dim), float(scale), float(diff)
+        self.norm_eps, self.window = float(norm_eps), int(window or 0)
+        self.position = position
+        self.rotary_dim = int(rotary_dim or 0) if position else 0
+        if self.rotary_dim % 2 or self.rotary_dim > self.head_dim:
+            raise PartError(f"differential_attention: {self.rotary_dim} rotated dimensions of a map of {self.head_dim}")
+        self.rope = None
+        self.w_in = self.w_o = None
+        self.lam = 0.0
+
+    def cache_spec(self):
+        return SharedValueKVCacheSpec(2 * self.num_kv_heads, self.head_dim, self.window, self.value_dim, self.num_kv_heads)
+
+    def bind(self, shared):
+        if self.position is not None:
+            if self.position not in shared:
+                raise PartError(f"differential_attention: the model has no position encoding named {self.position!r}")
+            self.rope = shared[self.position]
+            if getattr(self.rope, "rotary_dim", None) != self.rotary_dim or not hasattr(self.rope, "inv_freq"):
+                raise PartError(f"differential_attention: position encoding {self.position!r} must give the frequencies of "
+                                f"{self.rotary_dim} rotated dimensions")
+
+    def tensors(self):
+        h, nh, nkv, d, v = self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
+        t = {"q": TensorReq((nh * 2 * d, h), MATRIX), "k": TensorReq((nkv * 2 * d, h), MATRIX),
+             "v": TensorReq((nkv * v, h), MATRIX), "o": TensorReq((h, nh * v), MATRIX)}
+        t.update({n: TensorReq((d,), VECTOR) for n in ("lq1", "lk1", "lq2", "lk2")})
+        return t
+
+    @staticmethod
+    def _map_major(w, heads: int, d: int):
+        """Rows [head][map][d] -> [map][head][d]."""
+        return w.reshape(heads, 2, d, w.shape[1]).transpose(0, 1).reshape(heads * 2 * d, w.shape[1])
+
+    def load(self, tensors, dtype, device):
+        nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
+        rows = [self._map_major(tensors["q"], nh, d), self._map_major(tensors["k"], nkv, d), tensors["v"]]
+        self.w_in = K.prepare_weight(torch.cat(rows, dim=0).contiguous())
+        self.w_o = K.prepare_weight(tensors["o"])
+        dot = lambda a, b: float((tensors[a].double() * tensors[b].double()).sum().item())
+        self.lam = math.exp(dot("lq1", "lk1")) - math.exp(dot("lq2", "lk2")) + self.diff
+
+    def forward(self, x, step, cache, write_cache=True):
+        if not write_cache:
+            raise PartError("differential_attention: reads no other layer's cache")
+        nh, nkv, d, v = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
+        g = step.kv[cache.group]
+        p = K.linear(x, self.w_in)
+        freq = self.rope.inv_freq if self.rope is not None else None
+        nq, nk = 2 * nh * d, 2 * nkv * d
+        q = K.qkv_rope_prepare(p, 0, nq, nq + nk, freq, step.positions, g.slots, cache.k, cache.v, 2 * nh, 2 * nkv, nkv, d, v,
+                               self.rotary_dim, pairs=True)
+        a = K.attention_masked(q, cache.k, cache.v, g, step, self.window, 0, self.scale)
+        o = K.diff_combine(a, nh, self.lam, self.norm_eps, 1.0 - self.diff)
+        return K.linear(o, self.w_o, slices_ok=True)

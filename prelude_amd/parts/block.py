@@ -164,3 +164,50 @@ class SandwichNormMixerBlock(Block):
         y = self.mixer.forward(h, step, cache, write_cache)
         self.post_mixer_norm.forward_branch_then(y, residual, None, dtype)
         return None, residual
+
+
+@register_part("block", "parallel_branches")
+class ParallelBranchesBlock(Block):
+    """One norm, both branches on its output: h = norm(x), x <- x + (mixer(h) + ffn(h)).  The stream x is 32-bit and is
+    all that travels between such blocks (``hidden`` is handed on as None); the branches' outputs are added to each
+    other and then to the stream in 32-bit, in one launch."""
+    GRAPH_SAFE_PORTIONS = True
+    HANDS_ON_STREAM = True
+    LAUNCHES = 1
+
+    SLOTS = {"norm": "norm", "mixer": "mixer", "ffn": "ffn"}
+
+    def __init__(self, norm, mixer, ffn=None):
+        self.norm, self.mixer, self.ffn = norm, mixer, ffn
+
+    @staticmethod
+    def _enter(hidden, residual, step):
+        """(the stream, the engine's element type).  The first block turns the embedding into the stream (an embedding
+        that comes in 32-bit already is the stream)."""
+        if step.compute_dtype is None:
+            raise PartError("parallel_branches: the step does not say the engine's element type")
+        if residual is None:
+            hidden = K.as_tensor(hidden)
+            return (hidden if hidden.dtype == torch.float32 else K.to_f32(hidden)), step.compute_dtype
+        if residual.dtype != torch.float32 or hidden is not None:
+            raise PartError("parallel_branches: only a 32-bit stream travels between such blocks")
+        return residual, step.compute_dtype
+
+    def forward(self, hidden, residual, step, cache, write_cache=True):
+        residual, dtype = self._enter(hidden, residual, step)
+        h = self.norm.forward_stream(residual, dtype)
+        a = K.as_tensor(self.mixer.forward(h, step, cache, write_cache))
+        b = None
+        if self.ffn is not None:
+            b = K.as_tensor(self.ffn.forward(h, step=step) if getattr(self.ffn, "NEEDS_STEP", False) else self.ffn.forward(h))
+        K.stream_add_branches_(residual, a, b)
+        return None, residual
+
+
+@register_part("block", "parallel_branches_mixer_only")
+class ParallelBranchesMixerBlock(ParallelBranchesBlock):
+    """A ``parallel_branches`` layer without a feed-forward: x <- x + mixer(norm(x))."""
+    SLOTS = {"norm": "norm", "mixer": "mixer"}
+
+    def __init__(self, norm, mixer):
+        super().__init__(norm, mixer, None)

@@ -84,22 +84,36 @@ class RoutedExperts(FeedForward):
     LAUNCHES = 11
     GRAPH_SAFE_PORTIONS = True
 
-    def __init__(self, hidden_size: int, num_experts: int, top: int, expert_size: int, limit: float, route_scale: float = 1.0,
-                 alpha: float = 1.702, correction: bool = True, shared_size: int = 0, shared_limit: float = 0.0):
+    def __init__(self, hidden_size: int, num_experts: int, top: int, expert_size: int, limit: float = 0.0, route_scale: float = 1.0,
+                 alpha: float = 1.702, correction: bool = True, shared_size: int = 0, shared_limit: float = 0.0,
+                 activation: str = "clamped", router_bias: bool = False, route: str = "scores"):
+        """``activation``: ``"clamped"`` (the gated pair above) or ``"silu"`` (the plain gated pair silu(gate) * up, no
+        clamps), for the experts and the shared expert alike.  ``router_bias``: a stored vector ``router.b`` is added to
+        the router's logits.  ``route``: ``"scores"`` (above) or ``"chosen_logits"``: the ``top`` experts with the
+        largest logits, weighted by the softmax over those logits alone (no correction)."""
         if not 1 <= int(top) <= int(num_experts):
             raise PartError(f"routed_experts: {top} of {num_experts} experts a token")
-        if not limit > 0 or (shared_size and not shared_limit > 0):
+        if activation not in ("clamped", "silu"):
+            raise PartError(f"routed_experts: activation {activation!r} is not one of 'clamped', 'silu'")
+        if route not in ("scores", "chosen_logits"):
+            raise PartError(f"routed_experts: route {route!r} is not one of 'scores', 'chosen_logits'")
+        if route == "chosen_logits":
+            correction = False
+        if activation == "clamped" and (not limit > 0 or (shared_size and not shared_limit > 0)):
             raise PartError(f"routed_experts: the clamps {limit} and {shared_limit} must be positive")
+        self.activation, self.has_router_bias, self.route = activation, bool(router_bias), route
         self.hidden_size, self.num_experts, self.top = int(hidden_size), int(num_experts), int(top)
         self.expert_size, self.limit, self.alpha = int(expert_size), float(limit), float(alpha)
         self.route_scale, self.has_correction = float(route_scale), bool(correction)
         self.shared_size, self.shared_limit = int(shared_size or 0), float(shared_limit or 0.0)
-        self.router = self.correction = self.gate_up_t = self.down_t = None
+        self.router = self.correction = self.router_bias = self.gate_up_t = self.down_t = None
         self.shared_gate_up = self.shared_down = None
 
     def tensors(self):
         h, f, n = self.hidden_size, self.expert_size, self.num_experts
         t = {"router": TensorReq((n, h), MATRIX)}
+        if self.has_router_bias:
+            t["router.b"] = TensorReq((n,), VECTOR)
         if self.has_correction:
             t["correction"] = TensorReq((n,), VECTOR)
         for e in range(n):
@@ -122,6 +136,7 @@ class RoutedExperts(FeedForward):
         rows = [tensors["router"]] + ([tensors["shared.sg"]] if self.shared_size else [])
         self.router = torch.cat(rows, dim=0).contiguous()
         self.correction = tensors["correction"] if self.has_correction else None
+        self.router_bias = tensors["router.b"] if self.has_router_bias else None
         self.gate_up_t = K.GroupedWeight(torch.stack([self._pairs(tensors[f"e{e}.gate"], tensors[f"e{e}.up"]) for e in range(n)]))
         self.down_t = K.GroupedWeight(torch.stack([tensors[f"e{e}.down"] for e in range(n)]))
         if self.shared_size:
@@ -133,12 +148,18 @@ class RoutedExperts(FeedForward):
         # the router's sums and scores are 32-bit (the operands are of the engine's type): a product of few columns
         logits = K.linear_narrow_f32(x, self.router)
         choice, weights, gate = K.moe_route(logits, n, self.top, self.route_scale, self.correction,
-                                            gate_col=n if self.shared_size else -1)
+                                            gate_col=n if self.shared_size else -1, bias=self.router_bias,
+                                            by_logit=self.route == "chosen_logits")
         eo = K.moe_order(choice, n, self.top)
-        mid = K.moe_linear(x, self.gate_up_t, eo, from_tokens=True, clamped_gate_epilogue=(self.limit, self.alpha))
+        silu = self.activation == "silu"
+        if silu:
+            mid = K.moe_linear(x, self.gate_up_t, eo, from_tokens=True, silu_gate_epilogue=True)
+        else:
+            mid = K.moe_linear(x, self.gate_up_t, eo, from_tokens=True, clamped_gate_epilogue=(self.limit, self.alpha))
         y = K.moe_linear(mid, self.down_t, eo, from_tokens=False, out_dtype=torch.float32)
         base: Optional[torch.Tensor] = None
         if self.shared_size:
-            base = K.as_tensor(K.linear(K.linear_clamped_gate(x, self.shared_gate_up, self.shared_limit, self.alpha),
-                                        self.shared_down))
+            mid_s = K.linear_gated(x, self.shared_gate_up, "silu") if silu else \
+                K.linear_clamped_gate(x, self.shared_gate_up, self.shared_limit, self.alpha)
+            base = K.as_tensor(K.linear(mid_s, self.shared_down))
         return K.moe_combine(y, eo, 1.0, base, x.dtype, weights=weights, base_scale=gate)

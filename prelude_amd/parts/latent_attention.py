@@ -31,7 +31,7 @@ class LatentAttention(Mixer):
 
     def __init__(self, hidden_size: int, num_heads: int, head_dim: int, rot_dim: int, value_dim: int, kv_rank: int,
                  q_rank: int, norm_eps: float, scale: Optional[float] = None, position: Optional[str] = None,
-                 rotary_dim: Optional[int] = None, sink: bool = False, window: int = 0):
+                 rotary_dim: Optional[int] = None, sink: bool = False, window: int = 0, output_gate: bool = False):
         for name, v in (("hidden_size", hidden_size), ("num_heads", num_heads), ("head_dim", head_dim),
                         ("value_dim", value_dim), ("kv_rank", kv_rank), ("q_rank", q_rank)):
             if int(v) <= 0:
@@ -39,6 +39,9 @@ class LatentAttention(Mixer):
         self.hidden_size, self.num_heads, self.head_dim = int(hidden_size), int(num_heads), int(head_dim)
         self.rot_dim, self.value_dim, self.kv_rank, self.q_rank = int(rot_dim), int(value_dim), int(kv_rank), int(q_rank)
         self.norm_eps, self.window, self.sink = float(norm_eps), int(window or 0), bool(sink)
+        # the heads' outputs side by side times sigmoid(W_g x), element by element (tensor ``g`` [heads * value_dim,
+        # hidden]); the gate reads the mixer's input, as the projections do
+        self.output_gate = bool(output_gate)
         self.position = position
         self.rotary_dim = (self.rot_dim if rotary_dim is None else int(rotary_dim)) if position else 0
         if self.rot_dim < 0 or self.rotary_dim > self.rot_dim or self.rotary_dim % 2:
@@ -72,12 +75,15 @@ class LatentAttention(Mixer):
              "o": TensorReq((h, nh * v), MATRIX)}
         if self.sink:
             t["sink"] = TensorReq((nh,), VECTOR)
+        if self.output_gate:
+            t["g"] = TensorReq((nh * v, h), MATRIX)
         return t
 
     def load(self, tensors, dtype, device):
         nh, d, v, rank = self.num_heads, self.head_dim, self.value_dim, self.kv_rank
         # one product for both down projections: [q_rank | kv_rank | rot] rows
-        self.w_down = K.prepare_weight(torch.cat([tensors["dq"], tensors["dkv"]], dim=0).contiguous())
+        down = [tensors["dq"], tensors["dkv"]] + ([tensors["g"]] if self.output_gate else [])   # the gate's rows ride along
+        self.w_down = K.prepare_weight(torch.cat(down, dim=0).contiguous())
         self.w_uq = K.prepare_weight(tensors["uq"])
         self.w_o = K.prepare_weight(tensors["o"])
         # the per-head maps as [head, out, in]: W_uk[h] is [d, rank] as stored and is applied transposed (out rank,
@@ -92,14 +98,22 @@ class LatentAttention(Mixer):
         g = step.kv[cache.group]
         freq = self.rope.inv_freq if self.rope is not None else None
         down = K.linear(x, self.w_down)
+        gate = None
+        if self.output_gate:
+            gate = down[:, self.q_rank + rank + r:]
+            down = down[:, : self.q_rank + rank + r]
         cq = K.latent_prep(down, self.q_norm, self.c_norm, freq, step.positions, g.slots if write_cache else None,
                            cache.latent if write_cache else None, self.q_rank, rank, r, self.rotary_dim, self.norm_eps,
                            cache_t=cache.latent_t if write_cache else None)
         q = K.linear(cq, self.w_uq).view(-1, nh, d + r)
         ql = torch.empty((q.shape[0], nh, rank + r), dtype=q.dtype, device=q.device)
         K.head_linear(q, self.uk_t, ql)                                             # the key map, on the query side
-        K.rotate_pairs(q, ql, freq, step.positions, d, rank, r, self.rotary_dim)
+        if r:
+            K.rotate_pairs(q, ql, freq, step.positions, d, rank, r, self.rotary_dim)
         ol = K.latent_attention(ql, cache.latent, self.sinks, g, step, rank, self.window, self.scale, cache_t=cache.latent_t)
         o = torch.empty((q.shape[0], nh, v), dtype=q.dtype, device=q.device)
         K.head_linear(ol, self.uv_t, o)                                            # the value map, after the sum
-        return K.linear(o.view(-1, nh * v), self.w_o, slices_ok=True)
+        o = o.view(-1, nh * v)
+        if gate is not None:
+            o = K.sigmoid_gate(o, gate)
+        return K.linear(o, self.w_o, slices_ok=True)

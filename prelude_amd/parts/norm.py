@@ -88,17 +88,21 @@ class GroupRMSNorm(Norm):
     input through another norm of this kind)."""
     GRAPH_SAFE_PORTIONS = True
 
-    def __init__(self, size: int, eps: float, groups: int = 1):
+    def __init__(self, size: int, eps: float, groups: int = 1, scalar_weight: bool = False):
+        """``scalar_weight``: the stored weight is a single number for all coordinates (a tensor without axes)."""
         self.size, self.eps, self.groups = int(size), float(eps), int(groups)
         if self.groups < 1 or self.size % self.groups:
             raise PartError(f"group_rms_norm: {groups} groups do not divide a row of {size}")
+        self.scalar_weight = bool(scalar_weight)
         self.weight: Optional[torch.Tensor] = None
 
     def tensors(self):
-        return {"weight": TensorReq((self.size,), NORM)}
+        return {"weight": TensorReq(() if self.scalar_weight else (self.size,), NORM)}
 
     def load(self, tensors, dtype, device):
-        self.weight = tensors["weight"]
+        w = tensors["weight"]
+        # one number: spread over the row once, so that the kernels read a weight per coordinate as for any other norm
+        self.weight = w.reshape(1).expand(self.size).contiguous() if self.scalar_weight else w
 
     def as_rms(self):
         return (self.weight, self.eps) if self.groups == 1 else None
