@@ -212,3 +212,127 @@ def forward(cfg, w, tokens, streams=None):
     z = (rms_unit(x, cfg["norm"]["eps"]) * w["final.norm"]) @ w["head"].T
     cap = cfg.get("logit_softcap")
     return cap * np.tanh(z / cap) if cap else z
+
+
+# ---- configurations and weights of the tests' own --------------------------------------------------------------------------
+def _moe(ff, experts, top, shared):
+    m = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+    if shared:
+        m["shared"] = {"ff": shared}
+    return m
+
+
+def sink_layer(heads=4, kv_heads=2, dim=16, window=24, rot=8, base=10000.0, scale=0.25, mlp=None):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": scale, "mask": {"size": window}}
+    if rot:
+        m["rot"] = {"base": base, "dims": rot}
+    return {"type": "attention", "mixer": m, "mlp": mlp}
+
+
+def latent_layer(heads=3, dim=16, vdim=24, kv_rank=40, q_rank=24, window=20, scale=0.2, mlp=None):
+    return {"type": "latent_attention", "mlp": mlp,
+            "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "kv_rank": kv_rank, "q_rank": q_rank, "scale": scale,
+                      "mask": {"size": window}}}
+
+
+def diff_layer(heads=4, kv_heads=2, dim=8, vdim=24, window=18, rot=4, base=5000.0, scale=0.3, diff=0.25, mlp=None):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale, "diff": diff, "mask": {"size": window}}
+    if rot:
+        m["rot"] = {"base": base, "dims": rot}
+    return {"type": "attention_2", "mixer": m, "mlp": mlp}
+
+
+def model(layers, width=48, vocab=90, loop=None, taps=3, buckets=37, mul_prev=5, mul_cur=11, scale=3.0, cap=8.0, eps=1e-5):
+    cfg = {"architecture": "Nivasun", "vocab": vocab, "width": width, "norm": {"eps": eps}, "canon": {"taps": taps},
+           "embedding": {"scale": scale, "bigram": {"buckets": buckets, "mul_prev": mul_prev, "mul_cur": mul_cur}},
+           "layers": layers, "logit_softcap": cap}
+    if loop:
+        cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return cfg
+
+
+def tiny_config_p():
+    """Every mixer once, the two in the middle run three times; heads over fewer KV heads; three taps."""
+    return model([sink_layer(mlp=_moe(24, 6, 2, 40)), latent_layer(mlp=_moe(16, 4, 1, 0)), diff_layer(mlp=None),
+                  sink_layer(heads=2, kv_heads=1, dim=32, window=40, rot=32, mlp=_moe(24, 5, 5, 24))],
+                 loop=(1, 3, 3))
+
+
+def tiny_config_q():
+    """The whole model looped twice; heads of 64 (a size the matrix cores take); every expert chosen; two taps."""
+    return model([diff_layer(heads=2, kv_heads=2, dim=32, vdim=64, window=33, rot=16, mlp=_moe(32, 3, 3, 16)),
+                  sink_layer(heads=4, kv_heads=4, dim=64, window=70, rot=64, mlp=_moe(32, 8, 3, 16)),
+                  latent_layer(heads=2, dim=64, vdim=64, kv_rank=64, q_rank=32, window=50, mlp=_moe(32, 8, 2, 16))],
+                 width=64, vocab=120, loop=(0, 3, 2), taps=2, buckets=64, mul_prev=1, mul_cur=1, cap=30.0)
+
+
+def tiny_config_r():
+    """No loop, one tap (the convolution is a number a channel), no rotation anywhere, windows of one and two keys, a width that is
+    no whole 16-byte pieces."""
+    return model([latent_layer(heads=1, dim=8, vdim=8, kv_rank=12, q_rank=12, window=1, mlp=_moe(12, 2, 1, 12)),
+                  sink_layer(heads=3, kv_heads=3, dim=12, window=2, rot=0, mlp=None),
+                  diff_layer(heads=1, kv_heads=1, dim=12, vdim=12, window=64, rot=0, diff=0.6, mlp=_moe(12, 2, 2, 0))],
+                 width=36, vocab=50, loop=None, taps=1, buckets=7, mul_prev=0, mul_cur=3, cap=0.0)
+
+
+def tensor_shapes(cfg):
+    """Tensor name -> shape, as the design's files hold them."""
+    h, v = cfg["width"], cfg["vocab"]
+    t = {"embed": (v, h), "bigram": (cfg["embedding"]["bigram"]["buckets"] + 1, h), "final.norm": (), "head": (v, h)}
+    if cfg.get("loop"):
+        t["loop.step"] = (cfg["loop"]["times"], h)
+    for i, lc in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", lc["mixer"]
+        t[p + "norm1"] = ()
+        t[p + "canon1"] = (h, cfg["canon"]["taps"])
+        H, d = m["heads"], m["dim"]
+        if lc["type"] == "attention":
+            G = m["kv_heads"]
+            t.update({p + "mix.q": (H * d, h), p + "mix.k": (G * d, h), p + "mix.temp": (H,), p + "mix.sink": (H,),
+                      p + "mix.o": (h, H * d)})
+        elif lc["type"] == "latent_attention":
+            dv, r, rq = m["vdim"], m["kv_rank"], m["q_rank"]
+            t.update({p + "mix.dq": (rq, h), p + "mix.dq.norm": (rq,), p + "mix.uq": (H * d, rq), p + "mix.dkv": (r, h),
+                      p + "mix.dkv.norm": (r,), p + "mix.uk": (H * d, r), p + "mix.uv": (H * dv, r), p + "mix.g": (H * dv, h),
+                      p + "mix.o": (h, H * dv)})
+        else:
+            G, dv = m["kv_heads"], m["vdim"]
+            t.update({p + "mix.q": (H * 2 * d, h), p + "mix.k": (G * 2 * d, h), p + "mix.v": (G * dv, h), p + "mix.o": (h, H * dv)})
+            t.update({p + "mix." + n: (d,) for n in ("lq1", "lk1", "lq2", "lk2")})
+        f = lc.get("mlp")
+        if f:
+            ff, n = f["expert"]["ff"], f["router"]["experts"]
+            t.update({p + "mlp.router": (n, h), p + "mlp.router.b": (n,)})
+            for e in range(n):
+                t.update({f"{p}mlp.e{e}.gate": (ff, h), f"{p}mlp.e{e}.up": (ff, h), f"{p}mlp.e{e}.down": (h, ff)})
+            if f.get("shared"):
+                s = f["shared"]["ff"]
+                t.update({p + "mlp.shared.gate": (s, h), p + "mlp.shared.up": (s, h), p + "mlp.shared.down": (h, s),
+                          p + "mlp.shared.sg": (1, h)})
+    return t
+
+
+def random_weights(cfg, seed):
+    """Weights that bfloat16 holds exactly, as float64 arrays: matrices N(0, 1/sqrt(inputs)), norm weights and
+    temperatures around 1, sinks, router biases and the loop's vectors of a size that shows."""
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    w = {}
+    for name, shape in tensor_shapes(cfg).items():
+        last = name.rsplit(".", 1)[-1]
+        if last in ("norm1", "norm") or name.endswith(".temp"):
+            x = 1.0 + 0.2 * torch.randn(shape, generator=g)
+        elif last in ("sink", "b"):
+            x = 0.7 * torch.randn(shape, generator=g)
+        elif last in ("lq1", "lk1", "lq2", "lk2"):
+            x = 0.3 * torch.randn(shape, generator=g)
+        elif last == "canon1":
+            x = 0.4 * torch.randn(shape, generator=g)
+        elif name in ("loop.step", "bigram"):
+            x = 0.5 * torch.randn(shape, generator=g)
+        elif name == "embed":
+            x = 0.4 * torch.randn(shape, generator=g)
+        else:
+            x = torch.randn(shape, generator=g) / math.sqrt(shape[-1])
+        w[name] = x.to(torch.bfloat16).to(torch.float64).numpy()
+    return w
