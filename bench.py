@@ -162,6 +162,40 @@ def tedalix_record(args):
     return arch_record(args, "tedalix", (("tedalix", tedalix_shape(args.layers or 12)), ("fazopel_beside", fazopel_beside_tedalix(args.layers or 12))))
 
 
+# ``--arch nivasun``: a decoder of the Nivasun design at layer sizes of a real model of that kind: eight layers in periods
+# of four (attention with its keys for values, a temperature and a sink per head; two maps a head, one taken off the
+# other; attention through latents with an output gate; two maps again), every mixer behind a convolution over four
+# tokens and under a sliding window, routed experts with a gated shared one beside it on the same norm, the four layers
+# in the middle run twice (twelve runs) -- beside the closest existing design at equal size, a Fazopel decoder of twelve
+# attention layers (keys for values, a sink) with the same experts, width, vocabulary and head sizes
+def nivasun_shape(layers=8, width=2048, vocab=65536):
+    moe = dict(kind="moe", expert=dict(ff=1408), router=dict(experts=64, top=6), shared=dict(ff=2816))
+    sink = dict(heads=16, kv_heads=8, dim=128, vdim=128, scale=128 ** -0.5, mask=dict(size=1024), rot=dict(base=1000000.0, dims=64))
+    maps = dict(heads=16, kv_heads=8, dim=64, vdim=128, scale=64 ** -0.5, diff=0.35, mask=dict(size=512), rot=dict(base=10000.0, dims=64))
+    latent = dict(heads=16, dim=128, vdim=128, kv_rank=512, q_rank=768, scale=128 ** -0.5, mask=dict(size=1024))
+    period = (("attention", sink), ("attention_2", maps), ("latent_attention", latent), ("attention_2", maps))
+    start = min(2, layers)
+    return dict(architecture="Nivasun", vocab=vocab, width=width, norm=dict(eps=1e-6), canon=dict(taps=4),
+                embedding=dict(scale=width ** 0.5, bigram=dict(buckets=100003, mul_prev=36313, mul_cur=27191)),
+                layers=[dict(type=period[i % 4][0], mixer=period[i % 4][1], mlp=moe) for i in range(layers)],
+                loop=dict(start=start, stop=max(start, layers - 2), times=2), logit_softcap=30.0)
+
+
+def fazopel_beside_nivasun(runs=12):
+    raw = fazopel_shape(runs)
+    for lc in raw["layers"]:
+        lc["type"], lc["mixer"] = "attention", raw["layers"][3]["mixer"]
+        lc["mlp"] = raw["layers"][1]["mlp"]
+    return raw
+
+
+def nivasun_record(args):
+    """Prefill and decode throughput of the Nivasun shape and of an all-attention Fazopel shape beside it, same points."""
+    layers = args.layers or 8
+    runs = layers + max(0, layers - 2 - min(2, layers))
+    return arch_record(args, "nivasun", (("nivasun", nivasun_shape(layers)), ("fazopel_beside", fazopel_beside_nivasun(runs))))
+
+
 def build_engine(raw, dtype, cache_tokens, seed=0, page_size=16, **cfg_overrides):
     """The engine in its random-weights mode: the product's own loader, tensors drawn on the device."""
     from prelude_amd.config import EngineConfig
@@ -397,8 +431,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has (named in config)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--shape", default="4b", choices=sorted(SHAPES), help="layer sizes: Qwen3-4B (the default run), 0.6B, 8B or 32B")
-    ap.add_argument("--arch", default="qwen3", choices=["qwen3", "libodra", "fazopel", "tedalix"],
-                    help="libodra, fazopel, tedalix: prefill and decode of that design at a real model's layer sizes beside the closest other "
+    ap.add_argument("--arch", default="qwen3", choices=["qwen3", "libodra", "fazopel", "tedalix", "nivasun"],
+                    help="libodra, fazopel, tedalix, nivasun: prefill and decode of that design at a real model's layer sizes beside the closest other "
                          "decoder of equal size, as one record (the default run and its record are Qwen3's)")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the points at other batches and lengths")
@@ -430,6 +464,9 @@ def main() -> int:
         return 0
     if args.arch == "tedalix":
         print(json.dumps(tedalix_record(args)), flush=True)
+        return 0
+    if args.arch == "nivasun":
+        print(json.dumps(nivasun_record(args)), flush=True)
         return 0
     raw = dict(SHAPES[args.shape])
     name = f"Qwen3-{args.shape.upper()} shape"

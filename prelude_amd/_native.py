@@ -84,7 +84,7 @@ _KERNEL_API = {
     "pa_moe_linear": (I, [P, I, I, I, P, P, P, P, P, I, I, I, I, I, I, I]),
     "pa_moe_linear_mfma": (I, [P, I, P, P, P, P, P, I, I, I, I, I, I, I, F, F]),
     "pa_head_linear_mfma": (I, [P, P, P, P, I, I, I, I, c_long, c_long, c_long, c_long]),
-    "pa_moe_combine": (I, [P, I, P, P, P, F, P, P, P, I, I, I]),
+    "pa_moe_combine": (I, [P, I, P, P, P, F, P, P, P, I, I, I, P, P]),
     "pa_gemm_narrow": (I, [P, P, P, P, I, I, I, c_long, c_long]),
     "pa_moe_route": (I, [P, P, I, P, P, P, P, I, I, I, F, I, P, I]),
     "pa_qknorm_rope_kv_freq": (I, [P, I, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, P]),
@@ -115,7 +115,7 @@ _KERNEL_API = {
     "pa_gated_delta": (I, [P, P, P, P, P, P, P, P, I, I, I, I, I]),
     "pa_rotate_halves_f32": (I, [P, I, P, c_long, I, I, I, P, P, P, I, I, I, I, I, F]),
     "pa_pair_embed": (I, [P, I, P, P, P, P, P, P, P, P, P, I, I, I, I, c_long, c_long, F]),
-    "pa_time_conv_add": (I, [P, I, P, P, P, P, P, P, P, I, I, I, I]),
+    "pa_time_conv_add": (I, [P, I, P, P, P, P, P, P, P, I, I, I, I, I]),
     "pa_stream_add_row": (I, [P, P, P, I, I]),
     "pa_stream_add_branches": (I, [P, I, P, P, P, c_long]),
     "pa_qkv_rope_prepare": (I, [P, I, P, c_long, I, I, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I]),

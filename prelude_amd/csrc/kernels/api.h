@@ -266,8 +266,10 @@ int pa_moe_linear(void* stream, int x_dtype, int w_dtype, int y_dtype, const voi
                   const int* offsets, const int* order, int entries, int experts, int top, int K, int N, int from_tokens,
                   int act);
 // out[t] = (base_scale ? base_scale[t] : 1) * base[t] + sum_j w[t, j] * y[place[t * top + j]]
+// With `into` (a 32-bit stream [tokens, width]): into[t] += other[t] (or null) + that sum, unrounded, and nothing goes to out.
 int pa_moe_combine(void* stream, int dtype, const float* y, const int* place, const float* weights, float weight,
-                   const void* base, const float* base_scale, void* out, int tokens, int top, int width);
+                   const void* base, const float* base_scale, void* out, int tokens, int top, int width, float* into,
+                   const void* other);
 // A router: logits [tokens, ld] (32-bit; the first `experts` columns), s = softmax(logits); the `top` experts with the
 // largest s + correction[e] (correction null: none) -> choice [tokens, top]; weights [tokens, top] = their s over the
 // sum of the chosen s (+ 1e-20), times scale.  gate_out (or null) [tokens] = sigmoid(logits[t, gate_col]), a gate a
@@ -327,7 +329,8 @@ int pa_pair_embed(void* stream, int dtype, const int* ids, const int* positions,
                   const int* state_slots, int* prev_state, const void* table, const void* pair, float* out, int tokens,
                   int hidden, int vocab, int buckets, long mul_prev, long mul_cur, float scale);
 int pa_time_conv_add(void* stream, int dtype, const void* h, const float* w, float* state, const int* seq_of_token,
-                     const int* cu_q, const int* state_slots, void* out, int tokens, int nseq, int channels, int taps);
+                     const int* cu_q, const int* state_slots, void* out, int tokens, int nseq, int channels, int taps,
+                     int all_single);
 int pa_stream_add_row(void* stream, float* x, const float* row, int tokens, int hidden);
 int pa_stream_add_branches(void* stream, int dtype, float* x, const void* a, const void* b, long total);
 int pa_qkv_rope_prepare(void* stream, int dtype, const void* p, long stride, int q_off, int k_off, int v_off,

@@ -148,8 +148,9 @@ __device__ __forceinline__ void load_k_gap(const KeyWalk& w, int kept, int key0,
   }
 }
 
+// nv value heads in a page, of which this walk reads head vh (key head k goes with value head k mod nv).
 template <int VD>
-__device__ __forceinline__ VChunks v_chunks_gap(const KeyWalk& w, int kept, int key0, int g) {
+__device__ __forceinline__ VChunks v_chunks_gap(const KeyWalk& w, int kept, int key0, int g, int nv, int vh) {
   VChunks v;
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
@@ -157,7 +158,7 @@ __device__ __forceinline__ VChunks v_chunks_gap(const KeyWalk& w, int kept, int 
     if (c >= w.hi) c = (w.hi - 1) & ~3;
     else if (c + 3 < w.lo && c >= kept) c = kept > 0 ? (kept - 1) & ~3 : w.lo & ~3;
     const int page = w.table[c >> w.page_shift];
-    v.p[t] = w.vc + ((((size_t)page * w.nkv + w.kvh) * VD) << w.page_shift) + (c & w.page_mask);
+    v.p[t] = w.vc + ((((size_t)page * nv + vh) * VD) << w.page_shift) + (c & w.page_mask);
   }
   v.joined = w.page_shift >= 3 && __all(v.p[1] == v.p[0] + 4);
   return v;
@@ -168,9 +169,9 @@ __device__ __forceinline__ VChunks v_chunks_gap(const KeyWalk& w, int kept, int 
 template <int KD, int VD, int GT, typename Visible>
 __device__ __forceinline__ void attend32_masked(const KeyWalk& w, int kept, int key0, int g, int r, const KFrag<KD>& kf,
                                                 const bf16x8 (*qf)[KD / 32], const ScoreMap& sm, const float* bias, int my_pos,
-                                                bool masked, HeadState<VD>* st, Visible vis) {
+                                                bool masked, HeadState<VD>* st, Visible vis, int nv, int vh) {
   constexpr int OT = VD / 16;
-  const VChunks vch = v_chunks_gap<VD>(w, kept, key0, g);
+  const VChunks vch = v_chunks_gap<VD>(w, kept, key0, g, nv, vh);
   bf16x8 va[OT];
 #pragma unroll
   for (int t = 0; t < OT; ++t) va[t] = load_v(vch, 16 * t + r, w.page_shift);
@@ -244,6 +245,7 @@ struct MaskedArgs {
   const bf16* gate;         // [T, gate_stride], or null
   size_t gate_stride;
   float out_scale;
+  int nv;                   // value heads in a page: key head k goes with value head k mod nv
 };
 
 // Grid (tiles of 64 tokens, nkv * head groups, sequences); WAVES wavefronts: four, or eight for steps in which every
@@ -312,7 +314,7 @@ __global__ __launch_bounds__(WAVES* kWave, WAVES == 8 ? 1 : 2) void attn_masked_
       const KFrag<KD> kf = kf_next;
       const int key0 = key_of(i);
       if (i + 1 < n_steps) load_k_gap<KD>(w, kept, key_of(i + 1), g, r, kf_next);   // the next step's K rows, a step ahead
-      attend32_masked<KD, VD, GT>(w, kept, key0, g, r, kf, qf, a.sm, bias, my_pos, masked_at(key0), st, vis);
+      attend32_masked<KD, VD, GT>(w, kept, key0, g, r, kf, qf, a.sm, bias, my_pos, masked_at(key0), st, vis, a.nv, kvh % a.nv);
     }
     if (!qvalid) return;
     const size_t t = (size_t)(row0 + t0 + r);
@@ -336,7 +338,7 @@ __global__ __launch_bounds__(WAVES* kWave, WAVES == 8 ? 1 : 2) void attn_masked_
     const int key0 = key_of(i);
     KFrag<KD> kf;
     load_k_gap<KD>(w, kept, key0, g, r, kf);
-    attend32_masked<KD, VD, GT>(w, kept, key0, g, r, kf, qf, a.sm, bias, my_pos, true, st, vis);
+    attend32_masked<KD, VD, GT>(w, kept, key0, g, r, kf, qf, a.sm, bias, my_pos, true, st, vis, a.nv, kvh % a.nv);
   }
   if (r == 0) {
 #pragma unroll
@@ -426,7 +428,9 @@ using namespace pa;
 
 // Whether the matrix-core kernel takes bfloat16 keys of `hd`, values of `vd` and pages of `page_size`.
 extern "C" int pa_attn_masked_mfma_supports(int hd, int vd, int page_size) {
-  return hd == vd && (hd == 32 || hd == 64 || hd == 96 || hd == 128) && page_size >= 4 && (page_size & (page_size - 1)) == 0;
+  const bool same = hd == vd && (hd == 32 || hd == 64 || hd == 96 || hd == 128);
+  const bool twice = vd == 2 * hd && (hd == 32 || hd == 64);   // values twice as wide as the keys (two maps a head over one value)
+  return (same || twice) && page_size >= 4 && (page_size & (page_size - 1)) == 0;
 }
 
 extern "C" int pa_attn_masked(void* stream, int dtype, const void* q, const void* k_cache, const void* v_cache,
@@ -448,30 +452,32 @@ extern "C" int pa_attn_masked(void* stream, int dtype, const void* q, const void
   PA_REQUIRE(out_stride >= (long)nh * vd && (!gate || gate_stride >= nh), "attn_masked: output stride %ld or gate stride %ld "
              "too small for %d heads of %d", out_stride, gate_stride, nh, vd);
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == kBF16 && nv == nkv && pa_attn_masked_mfma_supports(hd, vd, page_size) && cu_q && context_lens && nseq > 0 && max_q_len > 0) {
+  if (dtype == kBF16 && pa_attn_masked_mfma_supports(hd, vd, page_size) && cu_q && context_lens && nseq > 0 && max_q_len > 0) {
     const int group = nh / nkv;
     // two heads a wavefront where the group is even: four leave a head of 128 no registers and measured slower
     const int gt = group % 2 == 0 ? 2 : 1;
     MaskedArgs a{(const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache, block_table, table_stride, cu_q, context_lens,
                  (bf16*)out, (size_t)out_stride, nh, nkv, __builtin_ctz(page_size), window, window > 0 ? keep_first : 0,
                  score_map(scale, softcap, sink), softcap > 0.f ? 1.0f : 1.0f / scale, slopes, (const bf16*)gate,
-                 (size_t)gate_stride, out_scale};
+                 (size_t)gate_stride, out_scale, nv};
     dim3 mgrid((max_q_len + 63) / 64, nkv * (group / gt), nseq);
     const bool singles = max_q_len == 1;
-#define PA_MASKED(D, GT)                                                                                      \
+#define PA_MASKED(D, V, GT)                                                                                   \
   do {                                                                                                        \
-    if (singles) hipLaunchKernelGGL((attn_masked_mfma_kernel<D, D, GT, 8>), mgrid, dim3(512), 0, st, a);       \
-    else hipLaunchKernelGGL((attn_masked_mfma_kernel<D, D, GT, 4>), mgrid, dim3(256), 0, st, a);               \
+    if (singles) hipLaunchKernelGGL((attn_masked_mfma_kernel<D, V, GT, 8>), mgrid, dim3(512), 0, st, a);       \
+    else hipLaunchKernelGGL((attn_masked_mfma_kernel<D, V, GT, 4>), mgrid, dim3(256), 0, st, a);               \
   } while (0)
-#define PA_MASKED_GT(D)              \
-  do {                               \
-    if (gt == 2) PA_MASKED(D, 2);    \
-    else PA_MASKED(D, 1);            \
+#define PA_MASKED_GT(D, V)              \
+  do {                                  \
+    if (gt == 2) PA_MASKED(D, V, 2);    \
+    else PA_MASKED(D, V, 1);            \
   } while (0)
-    if (hd == 32) PA_MASKED_GT(32);
-    else if (hd == 64) PA_MASKED_GT(64);
-    else if (hd == 96) PA_MASKED_GT(96);
-    else PA_MASKED_GT(128);
+    if (hd == 32 && vd == 32) PA_MASKED_GT(32, 32);
+    else if (hd == 32) PA_MASKED_GT(32, 64);
+    else if (hd == 64 && vd == 64) PA_MASKED_GT(64, 64);
+    else if (hd == 64) PA_MASKED_GT(64, 128);
+    else if (hd == 96) PA_MASKED_GT(96, 96);
+    else PA_MASKED_GT(128, 128);
 #undef PA_MASKED_GT
 #undef PA_MASKED
     return check_launch("attn_masked (matrix cores)");

@@ -225,7 +225,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ place,
                                                          const float* __restrict__ weights, float weight,
                                                          const T* __restrict__ base, const float* __restrict__ base_scale,
-                                                         T* __restrict__ out, int top, int width) {
+                                                         T* __restrict__ out, int top, int width, float* __restrict__ into,
+                                                         const T* __restrict__ other) {
   __shared__ int place_s[kCombineTop];
   __shared__ float weight_s[kCombineTop];
   const int t = blockIdx.x;
@@ -253,6 +254,11 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
     if (i >= width) continue;
     float v = s[c];
     if (base) v += base_scale ? bs * to_f32(base[(size_t)t * width + i]) : to_f32(base[(size_t)t * width + i]);
+    if (into) {   // the branches' sum first, then the stream: x + (other + this)
+      if (other) v += to_f32(other[(size_t)t * width + i]);
+      into[(size_t)t * width + i] += v;
+      continue;
+    }
     out[(size_t)t * width + i] = from_f32<T>(v);
   }
 }
@@ -318,16 +324,18 @@ extern "C" int pa_moe_route(void* stream, const float* logits, int ld, const flo
 }
 
 extern "C" int pa_moe_combine(void* stream, int dtype, const float* y, const int* place, const float* weights, float weight,
-                              const void* base, const float* base_scale, void* out, int tokens, int top, int width) {
+                              const void* base, const float* base_scale, void* out, int tokens, int top, int width, float* into,
+                              const void* other) {
   if (tokens == 0) return 0;
   PA_REQUIRE(tokens > 0 && top > 0 && width > 0, "moe_combine: bad sizes tokens=%d top=%d width=%d", tokens, top, width);
+  PA_REQUIRE(into || out, "moe_combine: nowhere to write");
   hipStream_t st = (hipStream_t)stream;
   if (dtype == kF32)
     hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(tokens, (width + 1023) / 1024), dim3(256), 0, st, y, place, weights, weight, (const float*)base,
-                       base_scale, (float*)out, top, width);
+                       base_scale, (float*)out, top, width, into, (const float*)other);
   else if (dtype == kBF16)
     hipLaunchKernelGGL(moe_combine_kernel<bf16>, dim3(tokens, (width + 1023) / 1024), dim3(256), 0, st, y, place, weights, weight, (const bf16*)base,
-                       base_scale, (bf16*)out, top, width);
+                       base_scale, (bf16*)out, top, width, into, (const bf16*)other);
   else
     return pa::fail("moe_combine: unknown element type code %d", dtype);
   return check_launch("moe_combine");

@@ -3,8 +3,8 @@
 //   pa_pair_embed          out[t] = table[id] * scale + pair[(prev * mul_prev + id * mul_cur) mod buckets], 32-bit; the
 //                          previous token of a portion's first token comes from a per-request slot, which then takes
 //                          the portion's last token; a sequence's first token reads row `buckets`
-//   pa_time_conv_add       out = h + conv(h): a causal convolution over time on each channel, the last taps - 1 inputs
-//                          carried per request
+//   pa_time_conv_add       out = h + conv(h): a causal convolution over time on each channel (weights [taps, channels]),
+//                          the last taps - 1 inputs carried per request
 //   pa_stream_add_row      x[t] += row, in place
 //   pa_stream_add_branches x += a + b, in place (b may be absent)
 //   pa_qkv_rope_prepare    queries, keys and values out of a merged projection: the first `rot` dimensions of every
@@ -53,34 +53,66 @@ __global__ __launch_bounds__(256) void pair_embed_kernel(const int* __restrict__
   }
 }
 
-// One thread a (token, channel).  state [slots, taps - 1, C] 32-bit: the inputs at the taps - 1 positions before the
-// portion's start, oldest first (zeros before the sequence's start).
-template <typename T>
+// state [slots, taps - 1, C] 32-bit: the inputs at the taps - 1 positions before the portion's start, oldest first (zeros
+// before the sequence's start).  A thread owns V consecutive channels of a token (V = 8: 16-byte pieces of bfloat16).  A
+// sequence that brings one token is the only reader of its slot, so its thread moves the carried inputs on itself;
+// portions leave that to time_conv_carry_kernel, which runs behind this one.
+constexpr int kConvMaxTaps = 17;
+
+template <typename T, int V>
 __global__ __launch_bounds__(256) void time_conv_add_kernel(const T* __restrict__ h, const float* __restrict__ w,
-                                                            const float* __restrict__ state, const int* __restrict__ seq_of_token,
+                                                            float* __restrict__ state, const int* __restrict__ seq_of_token,
                                                             const int* __restrict__ cu_q, const int* __restrict__ state_slots,
                                                             T* __restrict__ out, int C, int taps) {
+  typedef T vec_t __attribute__((ext_vector_type(V)));
   const int t = blockIdx.x;
-  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * V;
   if (c >= C) return;
   const int seq = seq_of_token[t];
-  const int rel = t - cu_q[seq];
+  const int begin = cu_q[seq];
+  const int rel = t - begin;
+  const bool single = cu_q[seq + 1] - begin == 1;
   const int keep = taps - 1;
-  const float* st = state + (size_t)state_slots[seq] * keep * C;
-  const float x = to_f32(h[(size_t)t * C + c]);
-  float acc = 0.f;
+  float* st = keep > 0 ? state + (size_t)state_slots[seq] * keep * C : nullptr;
+  const vec_t xv = *reinterpret_cast<const vec_t*>(h + (size_t)t * C + c);
+  float x[V], acc[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) x[e] = to_f32(xv[e]), acc[e] = 0.f;
   for (int j = 0; j < taps; ++j) {
     const int back = keep - j;   // the input `back` positions before this token
-    float v;
-    if (back == 0) v = x;
-    else if (rel - back >= 0) v = to_f32(h[(size_t)(t - back) * C + c]);
-    else v = st[(size_t)(rel - back + keep) * C + c];
-    acc = fmaf(w[(size_t)c * taps + j], v, acc);
+    float v[V];
+    if (back == 0) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) v[e] = x[e];
+    } else if (rel - back >= 0) {
+      const vec_t pv = *reinterpret_cast<const vec_t*>(h + (size_t)(t - back) * C + c);
+#pragma unroll
+      for (int e = 0; e < V; ++e) v[e] = to_f32(pv[e]);
+    } else {
+      const float* sp = st + (size_t)(rel - back + keep) * C + c;
+#pragma unroll
+      for (int e = 0; e < V; ++e) v[e] = sp[e];
+      if (single && j > 0) {     // one token: the place before this one takes what this place held
+        float* dp = st + (size_t)(j - 1) * C + c;
+#pragma unroll
+        for (int e = 0; e < V; ++e) dp[e] = v[e];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[e] = fmaf(w[(size_t)j * C + c + e], v[e], acc[e]);   // w [taps, C]: a tap's weights side by side
   }
-  out[(size_t)t * C + c] = from_f32<T>(x + acc);
+  if (single && keep > 0) {
+    float* dp = st + (size_t)(keep - 1) * C + c;
+#pragma unroll
+    for (int e = 0; e < V; ++e) dp[e] = x[e];
+  }
+  vec_t ov;
+#pragma unroll
+  for (int e = 0; e < V; ++e) ov[e] = from_f32<T>(x[e] + acc[e]);
+  *reinterpret_cast<vec_t*>(out + (size_t)t * C + c) = ov;
 }
 
-// A thread a (sequence, channel): it reads all it needs before it writes.
+// A thread a (sequence, channel) of the sequences that bring more than one token: it reads all it needs before it writes.
 template <typename T>
 __global__ __launch_bounds__(256) void time_conv_carry_kernel(const T* __restrict__ h, float* __restrict__ state,
                                                               const int* __restrict__ cu_q, const int* __restrict__ state_slots,
@@ -89,10 +121,10 @@ __global__ __launch_bounds__(256) void time_conv_carry_kernel(const T* __restric
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= C) return;
   const int begin = cu_q[seq], n = cu_q[seq + 1] - begin;
-  if (n <= 0) return;
+  if (n <= 1) return;
   const int keep = taps - 1;
   float* st = state + (size_t)state_slots[seq] * keep * C;
-  float fresh[16];
+  float fresh[kConvMaxTaps - 1];
   for (int i = 0; i < keep; ++i) {
     const int rel = n - keep + i;   // the step's token this place now holds, or an older input when negative
     fresh[i] = rel >= 0 ? to_f32(h[(size_t)(begin + rel) * C + c]) : st[(size_t)(i + n) * C + c];
@@ -105,12 +137,24 @@ __global__ void stream_add_row_kernel(float* __restrict__ x, const float* __rest
   if (i < total) x[i] += row[i % H];
 }
 
-template <typename T>
+// Four elements a thread where the size allows (V = 4), else one.
+template <typename T, int V>
 __global__ void stream_add_branches_kernel(float* __restrict__ x, const T* __restrict__ a, const T* __restrict__ b, size_t total) {
-  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  typedef float fvec_t __attribute__((ext_vector_type(V)));
+  const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
   if (i >= total) return;
-  const float y = b ? to_f32(a[i]) + to_f32(b[i]) : to_f32(a[i]);
-  x[i] += y;
+  const vec_t av = *reinterpret_cast<const vec_t*>(a + i);
+  fvec_t xv = *reinterpret_cast<fvec_t*>(x + i);
+  if (b) {
+    const vec_t bv = *reinterpret_cast<const vec_t*>(b + i);
+#pragma unroll
+    for (int e = 0; e < V; ++e) xv[e] += to_f32(av[e]) + to_f32(bv[e]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < V; ++e) xv[e] += to_f32(av[e]);
+  }
+  *reinterpret_cast<fvec_t*>(x + i) = xv;
 }
 
 constexpr int kPrepWaves = 4;
@@ -239,29 +283,34 @@ extern "C" int pa_pair_embed(void* stream, int dtype, const int* ids, const int*
 }
 
 extern "C" int pa_time_conv_add(void* stream, int dtype, const void* h, const float* w, float* state, const int* seq_of_token,
-                                const int* cu_q, const int* state_slots, void* out, int tokens, int nseq, int channels, int taps) {
+                                const int* cu_q, const int* state_slots, void* out, int tokens, int nseq, int channels, int taps,
+                                int all_single) {
   if (tokens == 0) return 0;
-  PA_REQUIRE(tokens > 0 && nseq > 0 && channels > 0 && taps >= 1 && taps <= 17, "time_conv_add: bad sizes tokens=%d sequences=%d "
-             "channels=%d taps=%d", tokens, nseq, channels, taps);
+  PA_REQUIRE(tokens > 0 && nseq > 0 && channels > 0 && taps >= 1 && taps <= kConvMaxTaps, "time_conv_add: bad sizes tokens=%d "
+             "sequences=%d channels=%d taps=%d", tokens, nseq, channels, taps);
   PA_REQUIRE(taps == 1 || state, "time_conv_add: %d taps need the carried inputs", taps);
   PA_REQUIRE((channels + 255) / 256 <= 65535, "time_conv_add: %d channels exceed the grid", channels);
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid(tokens, (channels + 255) / 256), cgrid(nseq, (channels + 255) / 256);
-  if (dtype == kF32) {
-    hipLaunchKernelGGL(time_conv_add_kernel<float>, grid, dim3(256), 0, st, (const float*)h, w, state, seq_of_token, cu_q,
-                       state_slots, (float*)out, channels, taps);
-    if (taps > 1)
-      hipLaunchKernelGGL(time_conv_carry_kernel<float>, cgrid, dim3(256), 0, st, (const float*)h, state, cu_q, state_slots,
-                         channels, taps);
-  } else if (dtype == kBF16) {
-    hipLaunchKernelGGL(time_conv_add_kernel<bf16>, grid, dim3(256), 0, st, (const bf16*)h, w, state, seq_of_token, cu_q,
-                       state_slots, (bf16*)out, channels, taps);
-    if (taps > 1)
-      hipLaunchKernelGGL(time_conv_carry_kernel<bf16>, cgrid, dim3(256), 0, st, (const bf16*)h, state, cu_q, state_slots,
-                         channels, taps);
-  } else {
-    return pa::fail("time_conv_add: unknown element type code %d", dtype);
-  }
+  const bool wide = channels % 8 == 0 && (reinterpret_cast<uintptr_t>(h) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+  const int per = wide ? 8 : 1;
+  dim3 grid(tokens, (channels / per + 255) / 256), cgrid(nseq, (channels + 255) / 256);
+  const int threads = channels / per >= 256 ? 256 : 64 * ((channels / per + 63) / 64);
+#define PA_CONV(T)                                                                                                              \
+  do {                                                                                                                          \
+    if (wide)                                                                                                                   \
+      hipLaunchKernelGGL((time_conv_add_kernel<T, 8>), grid, dim3(threads), 0, st, (const T*)h, w, state, seq_of_token, cu_q,    \
+                         state_slots, (T*)out, channels, taps);                                                                 \
+    else                                                                                                                        \
+      hipLaunchKernelGGL((time_conv_add_kernel<T, 1>), grid, dim3(threads), 0, st, (const T*)h, w, state, seq_of_token, cu_q,    \
+                         state_slots, (T*)out, channels, taps);                                                                 \
+    if (taps > 1 && !all_single)                                                                                                \
+      hipLaunchKernelGGL(time_conv_carry_kernel<T>, cgrid, dim3(256), 0, st, (const T*)h, state, cu_q, state_slots, channels,   \
+                         taps);                                                                                                 \
+  } while (0)
+  if (dtype == kF32) PA_CONV(float);
+  else if (dtype == kBF16) PA_CONV(bf16);
+  else return pa::fail("time_conv_add: unknown element type code %d", dtype);
+#undef PA_CONV
   return check_launch("time_conv_add");
 }
 
@@ -278,11 +327,17 @@ extern "C" int pa_stream_add_branches(void* stream, int dtype, float* x, const v
   if (total == 0) return 0;
   PA_REQUIRE(total > 0 && x && a, "stream_add_branches: bad size %ld", total);
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid((unsigned)((total + 255) / 256));
-  if (dtype == kF32)
-    hipLaunchKernelGGL(stream_add_branches_kernel<float>, grid, dim3(256), 0, st, x, (const float*)a, (const float*)b, (size_t)total);
+  const bool wide = total % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) == 0;
+  const long per = wide ? 4 : 1;
+  dim3 grid((unsigned)((total / per + 255) / 256));
+  if (dtype == kF32 && wide)
+    hipLaunchKernelGGL((stream_add_branches_kernel<float, 4>), grid, dim3(256), 0, st, x, (const float*)a, (const float*)b, (size_t)total);
+  else if (dtype == kF32)
+    hipLaunchKernelGGL((stream_add_branches_kernel<float, 1>), grid, dim3(256), 0, st, x, (const float*)a, (const float*)b, (size_t)total);
+  else if (dtype == kBF16 && wide)
+    hipLaunchKernelGGL((stream_add_branches_kernel<bf16, 4>), grid, dim3(256), 0, st, x, (const bf16*)a, (const bf16*)b, (size_t)total);
   else if (dtype == kBF16)
-    hipLaunchKernelGGL(stream_add_branches_kernel<bf16>, grid, dim3(256), 0, st, x, (const bf16*)a, (const bf16*)b, (size_t)total);
+    hipLaunchKernelGGL((stream_add_branches_kernel<bf16, 1>), grid, dim3(256), 0, st, x, (const bf16*)a, (const bf16*)b, (size_t)total);
   else
     return pa::fail("stream_add_branches: unknown element type code %d", dtype);
   return check_launch("stream_add_branches");

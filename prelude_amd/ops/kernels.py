@@ -1475,10 +1475,14 @@ def moe_linear(x: torch.Tensor, w: GroupedWeight, eo: ExpertOrder, from_tokens: 
 
 
 def moe_combine(y: torch.Tensor, eo: ExpertOrder, weight: float, base: Optional[torch.Tensor], out_dtype: torch.dtype,
-                weights: Optional[torch.Tensor] = None, base_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+                weights: Optional[torch.Tensor] = None, base_scale: Optional[torch.Tensor] = None,
+                into: Optional[torch.Tensor] = None, other: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """out[t] = b[t] * base[t] + sum_j w * y[place[t * top + j]] in ascending j; y float32 [entries, H]; ``weights``
-    float32 [entries] per entry, else ``weight`` for all; ``base_scale`` float32 [T] gives b, else 1."""
-    _dev(y, base, weights, base_scale)
+    float32 [entries] per entry, else ``weight`` for all; ``base_scale`` float32 [T] gives b, else 1.  With ``into`` (a
+    32-bit stream [T, H]) the sum is not rounded and written but added in place, ``into[t] += other[t] + sum`` (``other``
+    of ``out_dtype`` or None: another branch's output, added to this one first), and nothing is returned."""
+    _dev(y, base, weights, base_scale, into, other)
+    _f32(into, "stream")
     _f32(y, "expert outputs")
     _f32(weights, "entry weights")
     _f32(base_scale, "base scale")
@@ -1486,9 +1490,14 @@ def moe_combine(y: torch.Tensor, eo: ExpertOrder, weight: float, base: Optional[
     h = y.shape[1]
     if y.shape[0] != eo.entries or (base is not None and (tuple(base.shape) != (t, h) or base.dtype != out_dtype)):
         raise NativeError(f"moe_combine: y {tuple(y.shape)} / base {None if base is None else tuple(base.shape)}")
-    out = torch.empty((t, h), dtype=out_dtype, device=y.device)
+    if into is not None:
+        if tuple(into.shape) != (t, h) or (other is not None and (tuple(other.shape) != (t, h) or other.dtype != out_dtype)):
+            raise NativeError(f"moe_combine: stream {tuple(into.shape)} / other {None if other is None else tuple(other.shape)}")
+    elif other is not None:
+        raise NativeError("moe_combine: another branch's output goes with a stream to add to")
+    out = torch.empty((t, h), dtype=out_dtype, device=y.device) if into is None else None
     check(kernels().pa_moe_combine(_stream(), _CODES[out_dtype], _ptr(y), _ptr(eo.place), _ptr(weights), float(weight), _ptr(base),
-                                   _ptr(base_scale), _ptr(out), t, eo.top, h))
+                                   _ptr(base_scale), _ptr(out), t, eo.top, h, _ptr(into), _ptr(other)))
     return out
 
 
@@ -1836,21 +1845,24 @@ def pair_embed(ids: torch.Tensor, step, prev_state: torch.Tensor, table: torch.T
 
 
 def time_conv_add(h: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Tensor], step) -> torch.Tensor:
-    """h + conv(h) with conv(h)_t = sum_j w[:, j] h_(t - taps + 1 + j) over time within each sequence, zeros before its
-    start.  h [T, C]; ``weight`` float32 [C, taps]; ``state`` float32 [slots, taps - 1, C]: a request's last taps - 1
-    inputs, read for the places before the portion and moved on afterwards."""
+    """h + conv(h) with conv(h)_t = sum_j w[j] h_(t - taps + 1 + j) over time within each sequence, zeros before its
+    start.  h [T, C]; ``weight`` float32 [taps, C] (a tap's weights side by side: the stored [C, taps] transposed);
+    ``state`` float32 [slots, taps - 1, C]: a request's last taps - 1 inputs, read for the places before the portion and
+    moved on afterwards."""
     _dev(h, weight, state, step.seq_of_token, step.cu_q, step.state_slots)
     _f32(weight, "convolution weight")
     _f32(state, "carried inputs")
     t, c = h.shape
-    taps = weight.shape[1]
-    if weight.dim() != 2 or weight.shape[0] != c or not h.is_contiguous() or \
+    taps = weight.shape[0]
+    if weight.dim() != 2 or weight.shape[1] != c or not h.is_contiguous() or \
             (taps > 1 and (state is None or tuple(state.shape[1:]) != (taps - 1, c))):
         raise NativeError(f"time_conv_add: h {tuple(h.shape)} / weight {tuple(weight.shape)} / state "
                           f"{None if state is None else tuple(state.shape)}")
     out = torch.empty_like(h)
+    # a step of single tokens alone: every thread moves its sequence's carried inputs on itself, no second launch
     check(kernels().pa_time_conv_add(_stream(), _code(h), _ptr(h), _ptr(weight), _ptr(state), _ptr(step.seq_of_token), _ptr(step.cu_q),
-                                     _ptr(step.state_slots), _ptr(out), t, int(step.num_seqs), c, taps))
+                                     _ptr(step.state_slots), _ptr(out), t, int(step.num_seqs), c, taps,
+                                     1 if int(getattr(step, "max_q_len", 0)) == 1 else 0))
     return out
 
 

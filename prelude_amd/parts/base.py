@@ -257,6 +257,17 @@ class FeedForward(Part):
         residual, h = norm.forward_residual(x, residual)
         return residual, (self.forward(h, step=step) if self.NEEDS_STEP else self.forward(h))
 
+    def forward_into_stream(self, x, stream: torch.Tensor, other=None, step=None) -> None:
+        """stream += other + forward(x), in 32-bit and in place (``other``: another branch's output on the same input, or
+        None): what a block asks for whose branches are added to the stream together.  A feed-forward whose last kernel
+        can add into the stream itself does so here; this is the plain order."""
+        from ..ops import kernels as K
+        y = K.as_tensor(self.forward(x, step=step) if self.NEEDS_STEP else self.forward(x))
+        if other is None:
+            K.stream_add_branches_(stream, y)
+        else:
+            K.stream_add_branches_(stream, K.as_tensor(other), y)
+
 
 class Norm(Part):
     # True for a norm whose three methods also take a product that was left as partial sums of slices of its

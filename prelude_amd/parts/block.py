@@ -173,7 +173,6 @@ class ParallelBranchesBlock(Block):
     other and then to the stream in 32-bit, in one launch."""
     GRAPH_SAFE_PORTIONS = True
     HANDS_ON_STREAM = True
-    LAUNCHES = 1
 
     SLOTS = {"norm": "norm", "mixer": "mixer", "ffn": "ffn"}
 
@@ -197,10 +196,10 @@ class ParallelBranchesBlock(Block):
         residual, dtype = self._enter(hidden, residual, step)
         h = self.norm.forward_stream(residual, dtype)
         a = K.as_tensor(self.mixer.forward(h, step, cache, write_cache))
-        b = None
-        if self.ffn is not None:
-            b = K.as_tensor(self.ffn.forward(h, step=step) if getattr(self.ffn, "NEEDS_STEP", False) else self.ffn.forward(h))
-        K.stream_add_branches_(residual, a, b)
+        if self.ffn is None:
+            K.stream_add_branches_(residual, a)
+        else:   # the feed-forward's last kernel takes the mixer's output along into the stream where it can
+            self.ffn.forward_into_stream(h, residual, a, step=step)
         return None, residual
 
 

@@ -48,7 +48,7 @@ class ConvInputMixer(Mixer):
         return t
 
     def load(self, tensors, dtype, device):
-        self.weight = tensors["conv"].contiguous()
+        self.weight = tensors["conv"].t().contiguous()   # [taps, channels]: a tap's weights side by side
         self.inner.load({name[len("inner."):]: t for name, t in tensors.items() if name.startswith("inner.")}, dtype, device)
 
     def forward(self, x, step, cache, write_cache=True):

@@ -144,6 +144,13 @@ class RoutedExperts(FeedForward):
             self.shared_down = K.prepare_weight(tensors["shared.down"])
 
     def forward(self, x, step=None):
+        return self._run(x, None, None)
+
+    def forward_into_stream(self, x, stream, other=None, step=None):
+        """The kernel that adds up a token's experts adds the sum, unrounded, and ``other`` into the stream itself."""
+        self._run(x, stream, None if other is None else K.as_tensor(other))
+
+    def _run(self, x, stream, other):
         n = self.num_experts
         # the router's sums and scores are 32-bit (the operands are of the engine's type): a product of few columns
         logits = K.linear_narrow_f32(x, self.router)
@@ -162,4 +169,4 @@ class RoutedExperts(FeedForward):
             mid_s = K.linear_gated(x, self.shared_gate_up, "silu") if silu else \
                 K.linear_clamped_gate(x, self.shared_gate_up, self.shared_limit, self.alpha)
             base = K.as_tensor(K.linear(mid_s, self.shared_down))
-        return K.moe_combine(y, eo, 1.0, base, x.dtype, weights=weights, base_scale=gate)
+        return K.moe_combine(y, eo, 1.0, base, x.dtype, weights=weights, base_scale=gate, into=stream, other=other)

@@ -119,7 +119,7 @@ def test_time_convolution_carries_its_inputs_across_cuts(gpu, dtype, channels, t
         qn = [cuts[i][k] for i in live]
         h = torch.cat([seqs[i][fed[i]: fed[i] + cuts[i][k]] for i in live]).to(gpu)
         st = step_of([fed[i] + cuts[i][k] for i in live], qn, gpu, slots=[slots[i] for i in live])
-        out = K.time_conv_add(h, w.to(gpu), state, st)
+        out = K.time_conv_add(h, w.t().contiguous().to(gpu), state, st)
         at = 0
         for i, n in zip(live, qn):
             got[i].append(out[at: at + n].cpu())
