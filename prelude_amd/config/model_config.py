@@ -685,6 +685,7 @@ class NivasunConfig:
     loop_stop: int
     loop_times: int             # 1 with start == stop: no loop
     layers: Tuple[NivasunLayerConfig, ...]
+    has_loop: bool = False      # the configuration has a `loop` (its file then holds a vector per pass, also for an empty stretch)
 
     ARCH = "Nivasun"
     MIXERS = ("attention", "latent_attention", "attention_2")
@@ -782,4 +783,4 @@ class NivasunConfig:
                    taps=_positive(_obj(raw, "canon", a), "taps", int, a, "canon."),
                    embed_scale=_get(emb, "scale", float, a, default=1.0), buckets=_positive(pair, "buckets", int, a, pw),
                    mul_prev=_get(pair, "mul_prev", int, a), mul_cur=_get(pair, "mul_cur", int, a), logit_cap=cap,
-                   loop_start=start, loop_stop=stop, loop_times=times, layers=tuple(layers))
+                   loop_start=start, loop_stop=stop, loop_times=times, layers=tuple(layers), has_loop=loop is not None)

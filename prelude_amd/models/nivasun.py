@@ -97,7 +97,7 @@ def nivasun_spec(cfg: NivasunConfig) -> ModelSpec:
     h = cfg.width
     positions = {}
     layers = [_layer_spec(cfg, i, lc, positions) for i, lc in enumerate(cfg.layers)]
-    looped = cfg.loop_stop > cfg.loop_start
+    looped = cfg.has_loop   # a file of a configuration with a `loop` holds the passes' vectors, also where the stretch is empty
     return ModelSpec(
         architecture="Nivasun", vocab_size=cfg.vocab, hidden_size=h, max_positions=MAX_POSITIONS, eos_token_ids=(),
         embedding=PartSpec("pair_hash_embedding", dict(vocab_size=cfg.vocab, hidden_size=h, buckets=cfg.buckets,

@@ -46,6 +46,7 @@ def test_the_run_order_of_a_looped_stretch():
     empty = pn.tiny_config_r()
     empty["loop"] = {"start": 2, "stop": 2, "times": 4}
     assert [i for i, _ in run_order(NivasunConfig.from_dict(empty))] == [0, 1, 2]
+    assert build(empty).tensor_requests()["loop.step"].shape == (4, 36)     # the file holds them all the same
     tail = pn.tiny_config_r()
     tail["loop"] = {"start": 2, "stop": 3, "times": 2}
     assert run_order(NivasunConfig.from_dict(tail)) == [(0, None), (1, None), (2, 0), (2, 1)]

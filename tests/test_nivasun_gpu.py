@@ -694,3 +694,85 @@ def test_command_line_with_the_pools_sized_from_free_memory(gpu, capsys):
     assert cli.main(["--model", path, "--random-weights", "--prompt-len", "5", "--max-tokens", "3", "--max-cache-tokens", "256"]) == 0
     rec = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
     assert len(rec["token_ids"]) == 3 and all(0 <= t < cfg["vocab"] for t in rec["token_ids"])
+
+
+# ---- configurations drawn at random ------------------------------------------------------------------------------------
+def draw_config(seed):
+    """A Nivasun configuration drawn from a seed: any sizes the design allows, also ones no kernel is tuned for."""
+    rng = np.random.default_rng(seed)
+    pick = lambda xs: xs[int(rng.integers(0, len(xs)))]
+    window = lambda: int(pick([1, 2, 5, 16, 31, 32, 33, 64, 100]))
+
+    def mlp():
+        if rng.random() < 0.2:
+            return None
+        experts = int(pick([1, 2, 3, 5, 8, 16]))
+        return pn._moe(int(pick([8, 16, 24, 40, 64])), experts, int(rng.integers(1, experts + 1)), int(pick([0, 8, 24, 48])))
+
+    def rot(dim):
+        return int(pick([0, 2, dim // 2, dim])) // 2 * 2
+
+    layers = []
+    for _ in range(int(rng.integers(2, 6))):
+        kind = pick(["attention", "latent_attention", "attention_2"])
+        kv, group = int(pick([1, 2, 3])), int(pick([1, 2, 4]))
+        if kind == "attention":
+            dim = int(pick([8, 16, 24, 32, 64, 128]))
+            layers.append(pn.sink_layer(heads=kv * group, kv_heads=kv, dim=dim, window=window(), rot=rot(dim), base=float(pick([100.0, 1e4, 1e6])),
+                                        scale=float(pick([0.5, 1.0, 2.0])) / math.sqrt(dim), mlp=mlp()))
+        elif kind == "latent_attention":
+            dim = int(pick([8, 16, 32, 64]))
+            layers.append(pn.latent_layer(heads=kv * group, dim=dim, vdim=int(pick([8, 16, 24, 64])), kv_rank=int(pick([8, 12, 16, 40, 64, 96])),
+                                          q_rank=int(pick([8, 12, 24, 64])), window=window(), scale=float(pick([0.5, 1.0, 2.0])) / math.sqrt(dim), mlp=mlp()))
+        else:
+            dim = int(pick([8, 16, 32, 64]))
+            layers.append(pn.diff_layer(heads=kv * group, kv_heads=kv, dim=dim, vdim=2 * dim if rng.random() < 0.5 else int(pick([8, 16, 24, 40, 64])),
+                                        window=window(), rot=rot(dim), base=float(pick([100.0, 1e4, 5e4])), scale=float(pick([0.5, 1.0, 2.0])) / math.sqrt(dim),
+                                        diff=float(pick([0.0, 0.2, 0.5, 0.8])), mlp=mlp()))
+    n = len(layers)
+    loop = None
+    if rng.random() < 0.8:
+        start = int(rng.integers(0, n + 1))
+        loop = (start, int(rng.integers(start, n + 1)), int(pick([1, 2, 3])))
+    cfg = pn.model(layers, width=int(pick([32, 36, 48, 64, 72, 96, 128, 160])), vocab=int(rng.integers(40, 400)), loop=loop,
+                   taps=int(pick([1, 2, 3, 4, 5])), buckets=int(pick([1, 7, 64, 509, 4099])), mul_prev=int(pick([0, 1, 31, 1009])),
+                   mul_cur=int(pick([0, 1, 7, 997])), scale=float(pick([1.0, 4.0, 9.5])), cap=float(pick([0.0, 5.0, 15.0, 40.0])),
+                   eps=float(pick([1e-6, 1e-5, 1e-4])))
+    return cfg, int(pick([4, 8, 16, 32]))
+
+
+@pytest.mark.parametrize("seed", list(range(int(os.environ.get("PRELUDE_AMD_DRAWN_CONFIGS", "12")))))   # widen for a hunt
+def test_drawn_configuration(gpu, seed):
+    """Each drawn model whole, then in portions beside a request that decodes, through a pool and state slots that are
+    used again: in 32-bit as drawn, in bfloat16 with every expert chosen (see ``CONFIGS``)."""
+    from prelude_amd.trace import TraceRunner
+    rng = np.random.default_rng(2000 + seed)
+    for dtype in DTYPES:
+        cfg, page = draw_config(seed)
+        if dtype == "bfloat16":
+            for lc in cfg["layers"]:
+                if lc.get("mlp"):
+                    lc["mlp"]["router"]["top"] = lc["mlp"]["router"]["experts"]
+        toks = np.random.default_rng(2000 + seed).integers(0, cfg["vocab"], size=150).tolist()
+        other = np.random.default_rng(3000 + seed).integers(0, cfg["vocab"], size=40).tolist()
+        w = pn.random_weights(cfg, 300 + seed)
+        ref, ref_other = pn.forward(cfg, w, toks), pn.forward(cfg, w, other)
+        what = f"seed {seed} {dtype} page {page} {cfg}"
+        r = TraceRunner(write_model(cfg, w), dtype, 256, page_size=page, state_slots=2)
+        got = r.step([{"id": "w", "tokens": toks, "want": list(range(150))}], ["w"])
+        mostly(got, ref, dtype, "whole: " + what)
+        a, b, i, j = [], [], 0, 10
+        r.step([{"id": "o", "tokens": other[:10], "want": []}])
+        for n in (3, 70, 2, 17, 1, 1, 40, 16):
+            entries = [{"id": "p", "tokens": toks[i:i + n], "want": list(range(n))}]
+            if j < len(other):
+                entries.append({"id": "o", "tokens": [other[j]], "want": [0]})
+            out = r.step(entries)
+            a.append(out[:n])
+            if j < len(other):
+                b.append(out[n:])
+                j += 1
+            i += n
+        mostly(np.concatenate(a), ref[:i], dtype, "portions: " + what)
+        mostly(np.concatenate(b), ref_other[10:j], dtype, "decoding beside them: " + what)
+        assert r.engine.tables.audit() == ""
