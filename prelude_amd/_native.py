@@ -114,6 +114,7 @@ _KERNEL_API = {
     "pa_delta_prepare": (I, [P, I, P, c_long, I, I, P, I, P, P, P, P, P, c_long, I, P, P, P, P, P, I, I, I, I, I, I]),
     "pa_gated_delta": (I, [P, P, P, P, P, P, P, P, I, I, I, I, I]),
     "pa_rotate_halves_f32": (I, [P, I, P, c_long, I, I, I, P, P, P, I, I, I, I, I, F]),
+    "pa_latent_gather": (I, [P, I, P, P, I, P, P, P, I, I, I, I]),
     "pa_pair_embed": (I, [P, I, P, P, P, P, P, P, P, P, P, I, I, I, I, c_long, c_long, F]),
     "pa_time_conv_add": (I, [P, I, P, P, P, P, P, P, P, I, I, I, I, I]),
     "pa_stream_add_row": (I, [P, P, P, I, I]),

@@ -236,6 +236,10 @@ int pa_lightning_attn_chunked(void* stream, int dtype, const void* qkv, long ld,
 int pa_latent_prep(void* stream, int dtype, const void* in, const float* wq, const float* wc, const float* inv_freq,
                    const int* positions, const int* slots, void* cq_out, void* cache, void* cache_t, int page_size,
                    int tokens, int q_rank, int rank, int rot, int rot_dims, float eps, long in_stride);
+// out [rows, rank] = the first `rank` elements of the cached vectors [pages, page, width] at (seq[i], pos[i]) through the
+// block table: latents back out of their pages, for a product over them.
+int pa_latent_gather(void* stream, int dtype, const void* cache, const int* block_table, int table_stride, const int* seq,
+                     const int* pos, void* out, int rows, int rank, int width, int page_size);
 // in [tokens, heads, in_stride] -> out [tokens, heads, out_stride]: `width` elements from in_off to out_off of every
 // head, the first rot_dims of them rotated in pairs
 int pa_rotate_pairs(void* stream, int dtype, const void* in, void* out, const float* inv_freq, const int* positions,

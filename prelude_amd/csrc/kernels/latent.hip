@@ -25,6 +25,24 @@ namespace pa {
 constexpr int kLatMaxDk = 1024;   // rank + rot
 constexpr int kLatWaves = 4;
 
+template <typename T>
+__global__ __launch_bounds__(256) void latent_gather_kernel(const T* __restrict__ cache, const int* __restrict__ block_table,
+                                                            int table_stride, const int* __restrict__ seq, const int* __restrict__ pos,
+                                                            T* __restrict__ out, int rows, int rank, int width, int page_size) {
+  const int i = blockIdx.x * 4 + threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  if (i >= rows) return;
+  const int p = pos[i];
+  const int page = block_table[(size_t)seq[i] * table_stride + p / page_size];
+  const T* src = cache + ((size_t)page * page_size + p % page_size) * width;
+  T* dst = out + (size_t)i * rank;
+  if (sizeof(T) == 2 && rank % 8 == 0 && width % 8 == 0) {   // 16-byte pieces
+    typedef T vec_t __attribute__((ext_vector_type(8)));
+    for (int e = lane * 8; e < rank; e += kWave * 8) *reinterpret_cast<vec_t*>(dst + e) = *reinterpret_cast<const vec_t*>(src + e);
+  } else {
+    for (int e = lane; e < rank; e += kWave) dst[e] = src[e];
+  }
+}
+
 // ---- prep ------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void latent_prep_kernel(const T* __restrict__ in, const float* __restrict__ wq,
@@ -272,6 +290,18 @@ extern "C" int pa_latent_prep(void* stream, int dtype, const void* in, const flo
                                 inv_freq, positions, slots, (T*)cq_out, (T*)cache, (T*)cache_t, page_size, q_rank, rank, rot,
                                 rot_dims, eps, (size_t)in_stride));
   return check_launch("latent_prep");
+}
+
+// out[i, :] = the first `rank` elements of the cached vector of (seq[i], pos[i]); a wavefront a row.
+extern "C" int pa_latent_gather(void* stream, int dtype, const void* cache, const int* block_table, int table_stride, const int* seq,
+                                const int* pos, void* out, int rows, int rank, int width, int page_size) {
+  if (rows == 0) return 0;
+  PA_REQUIRE(rows > 0 && rank > 0 && rank <= width && page_size > 0 && table_stride > 0, "latent_gather: bad sizes rows=%d rank=%d "
+             "width=%d page=%d", rows, rank, width, page_size);
+  PA_BY_TYPE(dtype, "latent_gather",
+             hipLaunchKernelGGL(latent_gather_kernel<T>, dim3((rows + 3) / 4), dim3(256), 0, (hipStream_t)stream, (const T*)cache,
+                                block_table, table_stride, seq, pos, (T*)out, rows, rank, width, page_size));
+  return check_launch("latent_gather");
 }
 
 extern "C" int pa_rotate_pairs(void* stream, int dtype, const void* in, void* out, const float* inv_freq,

@@ -348,8 +348,8 @@ extern "C" int pa_qkv_rope_prepare(void* stream, int dtype, const void* p, long 
                                    void* q_out, void* k_cache, void* v_cache, int tokens, int nq, int nk, int nv, int hd, int vd,
                                    int rot, int pairs, int page_size) {
   if (tokens == 0) return 0;
-  PA_REQUIRE(tokens > 0 && nq > 0 && hd > 0 && hd <= kPrepMaxDim && p && q_out, "qkv_rope_prepare: bad sizes tokens=%d nq=%d hd=%d",
-             tokens, nq, hd);
+  PA_REQUIRE(tokens > 0 && nq >= 0 && hd > 0 && hd <= kPrepMaxDim && p && (q_out || nq == 0) && (nq > 0 || slots),
+             "qkv_rope_prepare: bad sizes tokens=%d nq=%d hd=%d", tokens, nq, hd);
   PA_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0 && (rot == 0 || (inv_freq && positions)),
              "qkv_rope_prepare: %d rotated dimensions of %d, or frequencies or positions missing", rot, hd);
   PA_REQUIRE(q_off >= 0 && q_off + (long)nq * hd <= stride, "qkv_rope_prepare: the queries do not fit the row of %ld", stride);

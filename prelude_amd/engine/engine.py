@@ -422,7 +422,7 @@ class Engine:
                          state_slots=view("state_slots"), fresh=view("fresh"), want_rows=view("want_rows"), kv=kv,
                          q_lens=counts, starts=list(starts), state_slots_host=state_host, fresh_host=fresh_host,
                          max_q_len=max(counts), max_context_len=stride * self.page_size if fixed else max(ends),
-                         page_size=self.page_size,
+                         page_size=self.page_size, graph=True if fixed else None,
                          decode_seqs=view("decode_seqs")[:len(dec)], prefill_seqs=view("prefill_seqs")[:len(pre)],
                          n_decode=len(dec), n_prefill=len(pre), max_prefill_q=max_pre,
                          # with fixed buffers the launch shapes must not follow the data.  The fewest tokens behind

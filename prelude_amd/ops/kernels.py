@@ -1327,6 +1327,21 @@ def head_linear(x: torch.Tensor, w: GroupedWeight, out: torch.Tensor, x_off: int
                                    x.shape[0], x.shape[1], k, n, *strides))
 
 
+def latent_gather(cache: torch.Tensor, block_table: torch.Tensor, seq: torch.Tensor, pos: torch.Tensor, rank: int) -> torch.Tensor:
+    """The latents of the cached positions (seq[i], pos[i]) back out of their pages, [N, rank]: the first ``rank``
+    elements of each cached vector (``cache`` [pages, page, width])."""
+    _dev(cache, block_table, seq, pos)
+    _i32(block_table, "block_table")
+    _i32(seq, "sequences")
+    _i32(pos, "positions")
+    if cache.dim() != 3 or not 0 < rank <= cache.shape[2] or seq.shape != pos.shape or seq.dim() != 1 or block_table.dim() != 2:
+        raise NativeError(f"latent_gather: cache {tuple(cache.shape)} / rank {rank} / rows {tuple(seq.shape)}")
+    out = torch.empty((seq.shape[0], rank), dtype=cache.dtype, device=cache.device)
+    check(kernels().pa_latent_gather(_stream(), _code(cache), _ptr(cache), _ptr(block_table), block_table.shape[1], _ptr(seq), _ptr(pos),
+                                     _ptr(out), seq.shape[0], int(rank), cache.shape[2], cache.shape[1]))
+    return out
+
+
 def latent_attention_generic(q: torch.Tensor, cache: torch.Tensor, sink: Optional[torch.Tensor], block_table: torch.Tensor,
                              seq_of_token: torch.Tensor, positions: torch.Tensor, rank: int, window: int,
                              scale: float) -> torch.Tensor:
@@ -1709,6 +1724,11 @@ def qkv_prepare(p: torch.Tensor, q_off: int, k_off: int, v_off: int, q_weight: O
     return q
 
 
+def attention_masked_mfma_supported(hd: int, vd: int, page_size: int) -> bool:
+    """Whether ``attention_masked`` runs these widths on the matrix cores (bfloat16)."""
+    return bool(kernels().pa_attn_masked_mfma_supports(int(hd), int(vd), int(page_size)))
+
+
 def attention_masked(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, group, step, window: int, keep_first: int,
                      scale: float, softcap: float = 0.0, slopes: Optional[torch.Tensor] = None,
                      sink: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
@@ -1914,7 +1934,7 @@ def qkv_rope_prepare(p: torch.Tensor, q_off: int, k_off: int, v_off: int, inv_fr
             raise NativeError(f"qkv_rope_prepare: caches {None if k_cache is None else tuple(k_cache.shape)} / "
                               f"{None if v_cache is None else tuple(v_cache.shape)} for {nk} key heads of {hd} and {nv} value heads of {vd}")
         page = k_cache.shape[2]
-    q = torch.empty((t, nq, hd), dtype=p.dtype, device=p.device)
+    q = torch.empty((t, nq, hd), dtype=p.dtype, device=p.device) if nq else None   # no query heads: keys and values alone
     if t:
         caching = slots is not None
         check(kernels().pa_qkv_rope_prepare(_stream(), _code(p), p.data_ptr(), p.stride(0), int(q_off), int(k_off), int(v_off),

@@ -403,6 +403,42 @@ def test_the_window_on_the_matrix_cores(gpu, make, over, decoded):
     assert got > 0 and abs(got - moved) <= 0.5 * moved + 0.03 * float(ref.std()), f"token {c} is inside what {i} sees: {got} against {moved}"
 
 
+@pytest.mark.parametrize("over,page", [(dict(heads=2, dim=64, vdim=64, kv_rank=64, q_rank=32, window=70), 16),
+                                       (dict(heads=3, dim=32, vdim=64, kv_rank=40, q_rank=24, window=33), 8),
+                                       (dict(heads=1, dim=128, vdim=128, kv_rank=96, q_rank=64, window=200), 16)])
+def test_long_portions_attend_through_expanded_latents(gpu, over, page, monkeypatch):
+    """Under the bfloat16 engine a long portion has every head's keys and values made from the latents it can see, in
+    temporary pages, where short ones and single tokens attend to the latents themselves.  Both against the plain
+    logits: whole, a long portion behind a prefix that ends inside a page (its window reaches back into the prefix), a long
+    portion beside a sequence that decodes, and the same prompt with the expanded form switched off."""
+    from prelude_amd.parts.latent_attention import LatentAttention
+    from prelude_amd.trace import TraceRunner
+    cfg = pn.model([pn.latent_layer(**over)], loop=(0, 1, 2), width=64)
+    w = pn.random_weights(cfg, 80)
+    toks, other = tokens(cfg, 700, 81), tokens(cfg, 60, 82)
+    ref, ref_other = pn.forward(cfg, w, toks), pn.forward(cfg, w, other)
+    path = write_model(cfg, w)
+    used = []
+    real = LatentAttention._expanded
+    monkeypatch.setattr(LatentAttention, "_expanded", lambda self, *a: used.append(1) or real(self, *a))
+    monkeypatch.setattr(LatentAttention, "EXPAND_FROM_TOKENS", 100)
+    r = TraceRunner(path, "bfloat16", 1024, page_size=page, state_slots=2)
+    mostly(r.step([{"id": "w", "tokens": toks, "want": list(range(700))}], ["w"]), ref, "bfloat16", "whole")
+    assert len(used) == 2, "both runs of the layer expanded"
+    outs = [r.step([{"id": "p", "tokens": toks[:53], "want": list(range(53))}])]
+    assert len(used) == 2, "a short portion attends to the latents themselves"
+    r.step([{"id": "o", "tokens": other[:40], "want": []}])
+    outs.append(r.step([{"id": "p", "tokens": toks[53:400], "want": list(range(347))}]))
+    both = r.step([{"id": "p", "tokens": toks[400:], "want": list(range(300))}, {"id": "o", "tokens": [other[40]], "want": [0]}])
+    assert len(used) == 6
+    mostly(np.concatenate(outs + [both[:300]]), ref, "bfloat16", "portions behind a prefix")
+    mostly(both[300:], ref_other[40:41], "bfloat16", "a single token beside a long portion")
+    monkeypatch.setattr(LatentAttention, "EXPAND_FROM_TOKENS", 1 << 30)
+    r2 = TraceRunner(path, "bfloat16", 1024, page_size=page, state_slots=1)
+    mostly(r2.step([{"id": "w", "tokens": toks, "want": list(range(700))}], ["w"]), ref, "bfloat16", "without the expanded form")
+    assert len(used) == 6
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_a_sink_and_a_temperature_show(gpu, dtype):
     """Sinks far above the scores in every other head (those heads all but vanish, also at the first token, where a
