@@ -778,10 +778,13 @@ def draw_config(seed):
 
 
 @pytest.mark.parametrize("seed", list(range(int(os.environ.get("PRELUDE_AMD_DRAWN_CONFIGS", "12")))))   # widen for a hunt
-def test_drawn_configuration(gpu, seed):
+def test_drawn_configuration(gpu, seed, monkeypatch):
     """Each drawn model whole, then in portions beside a request that decodes, through a pool and state slots that are
-    used again: in 32-bit as drawn, in bfloat16 with every expert chosen (see ``CONFIGS``)."""
+    used again: in 32-bit as drawn, in bfloat16 with every expert chosen (see ``CONFIGS``) and with portions of 64 tokens
+    or more attending through expanded latents where the drawn head sizes allow it."""
+    from prelude_amd.parts.latent_attention import LatentAttention
     from prelude_amd.trace import TraceRunner
+    monkeypatch.setattr(LatentAttention, "EXPAND_FROM_TOKENS", 64)
     rng = np.random.default_rng(2000 + seed)
     for dtype in DTYPES:
         cfg, page = draw_config(seed)
