@@ -770,11 +770,14 @@ class NivasunConfig:
         emb = _obj(raw, "embedding", a)
         pair = _obj(emb, "bigram", a, "embedding.")
         pw = "embedding.bigram."
-        for key in ("mul_prev", "mul_cur"):
-            try:
-                _get(pair, key, int, a)
-            except ConfigError as e:
-                raise ConfigError(str(e).replace(f"`{key}`", f"`{pw}{key}`")) from None
+        mul = {}
+        for key in ("mul_prev", "mul_cur"):   # any integers, also negative ones: the row is the sum modulo the buckets
+            v = pair.get(key)
+            if v is None:
+                raise ConfigError(f"failed to parse {a} config: missing required key `{pw}{key}`")
+            if isinstance(v, bool) or not isinstance(v, int):
+                raise ConfigError(f"failed to parse {a} config: `{pw}{key}` must be an integer, got {v!r}")
+            mul[key] = int(v)
         cap = _get(raw, "logit_softcap", float, a, default=0.0)
         if cap < 0:
             raise ConfigError(f"failed to parse {a} config: `logit_softcap` must not be negative, got {cap!r}")
@@ -782,5 +785,5 @@ class NivasunConfig:
                    norm_eps=_positive(_obj(raw, "norm", a), "eps", float, a, "norm."),
                    taps=_positive(_obj(raw, "canon", a), "taps", int, a, "canon."),
                    embed_scale=_get(emb, "scale", float, a, default=1.0), buckets=_positive(pair, "buckets", int, a, pw),
-                   mul_prev=_get(pair, "mul_prev", int, a), mul_cur=_get(pair, "mul_cur", int, a), logit_cap=cap,
+                   mul_prev=mul["mul_prev"], mul_cur=mul["mul_cur"], logit_cap=cap,
                    loop_start=start, loop_stop=stop, loop_times=times, layers=tuple(layers), has_loop=loop is not None)

@@ -32,7 +32,8 @@ class TokenEmbedding(Part):
 
 @register_part("embedding", "pair_hash_embedding")
 class PairHashEmbedding(Part):
-    """x = table[token] * scale + pair[(previous token * mul_prev + token * mul_cur) mod buckets], taken in 32-bit and
+    """x = table[token] * scale + pair[(previous token * mul_prev + token * mul_cur) mod buckets] (the modulus that is
+    never negative, whatever the multipliers' signs), taken in 32-bit and
     handed on as the 32-bit stream; a sequence's first token reads row ``buckets`` (the last) of the pair table.  The
     previous token is part of a request's state: an embedding that says ``NEEDS_STEP`` is called with the step and with
     the storage of its ``cache_spec()``, one int32 a request here."""
@@ -40,8 +41,8 @@ class PairHashEmbedding(Part):
     NEEDS_STEP = True
 
     def __init__(self, vocab_size: int, hidden_size: int, buckets: int, mul_prev: int, mul_cur: int, scale: float = 1.0):
-        if int(buckets) < 1 or int(mul_prev) < 0 or int(mul_cur) < 0:
-            raise PartError(f"pair_hash_embedding: {buckets} buckets, multipliers {mul_prev} and {mul_cur}")
+        if int(buckets) < 1:
+            raise PartError(f"pair_hash_embedding: {buckets} buckets")
         self.vocab_size, self.hidden_size, self.buckets = int(vocab_size), int(hidden_size), int(buckets)
         self.mul_prev, self.mul_cur, self.scale = int(mul_prev), int(mul_cur), float(scale)
         self.weight = self.pair = None

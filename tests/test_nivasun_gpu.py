@@ -70,7 +70,7 @@ def step_of(ctx, qn, gpu, slots=None, page=8):
 
 # ---- the embedding: a row by the token and the one before it; the token before a portion lives in a slot ------------------
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("hidden,buckets,mp,mc", [(48, 37, 5, 11), (320, 1, 3, 2), (100, 64, 0, 1), (36, 1000, 70001, 99991)])
+@pytest.mark.parametrize("hidden,buckets,mp,mc", [(48, 37, 5, 11), (320, 1, 3, 2), (100, 64, 0, 1), (36, 1000, 70001, 99991), (64, 53, -7, 3)])
 def test_pair_embedding_through_portions_and_slots(gpu, dtype, hidden, buckets, mp, mc):
     from prelude_amd.ops import kernels as K
     vocab = 75
